@@ -10,7 +10,7 @@ from typing import List, Optional
 @dataclass
 class ModelConfig:
     name: str = "llama"
-    architecture: str = "llama"   # llama | opt | qwen2 | qwen2_vl | pugovik | dunusun
+    architecture: str = "llama"   # llama | opt | qwen2 | qwen2_vl | pugovik | dunusun | tosipel
     vocab_size: int = 128256
     hidden_size: int = 4096
     intermediate_size: int = 14336
@@ -110,9 +110,11 @@ PRESETS = {
 class HybridLayerConfig:
     """One layer of a hybrid stack: which sequence mixer it has, the
     mixer's sizes and constants, and its feed-forward (None = no FF)."""
-    type: str                      # latent_attention | lightning
+    type: str                      # latent_attention | lightning | ...
     mixer: dict = field(default_factory=dict)
     mlp: Optional[dict] = None
+    # index of the layer whose tensors this layer uses (None: its own)
+    weights_of: Optional[int] = None
 
 
 @dataclass
@@ -213,6 +215,62 @@ def dunusun_from_dict(d: dict, name: str = "dunusun",
         logit_softcap=float(cap) if cap else None, model_dir=model_dir)
 
 
+@dataclass
+class TosipelConfig(ModelConfig):
+    """Tosipel: layers of windowed softmax attention with a sink (`attention`),
+    latent attention without positions (`latent_attention`) or a gated delta
+    rule recurrence (`delta`); the sublayers read the residual as it is and
+    only their output is RMS-normed; dense GELU-gated feed-forwards; a layer
+    may use another layer's weights with a cache of its own."""
+    layers: List[HybridLayerConfig] = field(default_factory=list)
+    embed_scale: float = 1.0
+    model_dir: Optional[str] = None     # weights live here (None = random)
+
+    @property
+    def weight_layers(self) -> List[int]:
+        """For every layer the index of the layer that owns its tensors."""
+        return [i if l.weights_of is None else l.weights_of
+                for i, l in enumerate(self.layers)]
+
+    @property
+    def has_recurrent_state(self) -> bool:
+        return any(l.type == "delta" for l in self.layers)
+
+
+def tosipel_from_dict(d: dict, name: str = "tosipel",
+                      model_dir: Optional[str] = None) -> TosipelConfig:
+    layers = [HybridLayerConfig(type=l["type"], mixer=dict(l["mixer"]),
+                                mlp=l.get("mlp"),
+                                weights_of=l.get("weights_of"))
+              for l in d["layers"]]
+    for i, l in enumerate(layers):
+        if l.type not in ("attention", "latent_attention", "delta"):
+            raise ValueError(f"layer {i}: unknown mixer type {l.type!r}")
+        if l.mlp is not None and l.mlp.get("kind", "dense") != "dense":
+            raise ValueError(f"layer {i}: unknown feed-forward kind")
+    for i, l in enumerate(layers):
+        seen = {i}
+        while l.weights_of is not None:       # follow a chain to its owner
+            j = int(l.weights_of)
+            if not 0 <= j < len(layers) or j in seen:
+                raise ValueError(f"layer {i}: bad weights_of {j}")
+            seen.add(j)
+            owner = layers[j]
+            if owner.type != layers[i].type:
+                raise ValueError(f"layer {i}: weights_of {j} is another "
+                                 "kind of layer")
+            if owner.weights_of is None:
+                layers[i].weights_of = j
+                break
+            l = owner
+    return TosipelConfig(
+        name=name, architecture="tosipel", vocab_size=int(d["vocab"]),
+        hidden_size=int(d["width"]), num_layers=len(layers),
+        rms_eps=float(d["norm"]["eps"]),
+        embed_scale=float((d.get("embedding") or {}).get("scale", 1.0)),
+        max_position=1 << 20, layers=layers, model_dir=model_dir)
+
+
 def load_model_dir(path: str) -> ModelConfig:
     """Read <path>/config.json and pick the config class by its
     `architecture` field."""
@@ -225,6 +283,9 @@ def load_model_dir(path: str) -> ModelConfig:
     if arch == "dunusun":
         return dunusun_from_dict(d, name=os.path.basename(
             os.path.normpath(path)) or "dunusun", model_dir=path)
+    if arch == "tosipel":
+        return tosipel_from_dict(d, name=os.path.basename(
+            os.path.normpath(path)) or "tosipel", model_dir=path)
     raise ValueError(f"{path}: unsupported architecture "
                      f"{d.get('architecture')!r}")
 
@@ -320,6 +381,50 @@ PRESETS.update({
     # bench stacks at the width of real deployments (random weights)
     "dunusun-2k": _dunusun_preset("dunusun-2k", 2048, 8),
     "dunusun-4k": _dunusun_preset("dunusun-4k", 4096, 8),
+})
+
+
+def _tosipel_preset(name, width, n_layers, vocab=32000, head=128, window=1024,
+                    kv_rank=512, q_rank=None, share=True):
+    """Synthetic Tosipel stacks for benchmarks: two delta-rule layers, one
+    windowed attention layer and one latent attention layer per group of
+    four; the second attention layer reuses the first one's weights."""
+    heads = max(width // head, 1)
+    ff = dict(kind="dense", ff=3 * width // 2)
+    layers, first_attn = [], None
+    for i in range(n_layers):
+        k = i % 4
+        if k == 1:
+            lc = dict(type="attention", mlp=ff, mixer=dict(
+                heads=heads, kv_heads=max(heads // 4, 1), dim=head, vdim=head,
+                mask=dict(size=window), rot=dict(base=10000.0, dims=head // 2),
+                scale=head ** -0.5))
+            if first_attn is None:
+                first_attn = i
+            elif share:
+                lc["weights_of"] = first_attn
+            layers.append(lc)
+        elif k == 3:
+            layers.append(dict(type="latent_attention", mlp=ff, mixer=dict(
+                heads=heads, dim=head, vdim=head, kv_rank=kv_rank,
+                q_rank=q_rank or max(width // 2, 16), scale=head ** -0.5)))
+        else:
+            layers.append(dict(type="delta", mlp=ff, mixer=dict(
+                heads=heads, kv_heads=max(heads // 2, 1), dim=head, vdim=head,
+                conv=4)))
+    return tosipel_from_dict(dict(
+        architecture="Tosipel", vocab=vocab, width=width, layers=layers,
+        norm=dict(eps=1e-6), embedding=dict(scale=float(width) ** 0.5)),
+        name=name)
+
+
+PRESETS.update({
+    # CPU-test sized stack (the second attention layer shares weights)
+    "tosipel-tiny": _tosipel_preset("tosipel-tiny", 64, 6, vocab=256, head=16,
+                                    window=24, kv_rank=24, q_rank=20),
+    # bench stacks at the width of real deployments (random weights)
+    "tosipel-2k": _tosipel_preset("tosipel-2k", 2048, 8),
+    "tosipel-4k": _tosipel_preset("tosipel-4k", 4096, 8),
 })
 
 

@@ -22,6 +22,15 @@ GatedLinearAttention   S <- diag(alpha) S + k v^T, o = S^T q with a low-rank
                        per head, SiLU gate.
 ParallelMixer          two mixers reading the same input, outputs added
                        with fixed weights.
+SinkWindowAttention    softmax attention with grouped key/value heads over a
+                       sliding window of keys, RMS norm over the whole query
+                       and key projection, rotate-half positions on part of
+                       each head, a learned per-head sink in the softmax
+                       denominator, one sigmoid gate number per head.
+GatedDeltaRule         S <- g S; u = beta (v - S^T k); S <- S + k u^T;
+                       o = S^T q with unit q, k after a short convolution and
+                       SiLU; per-head scalar decay g; RMS norm per head, SiLU
+                       gate.
 
 All take the slice of a merged input projection that belongs to them and
 return the mixer output in the model dtype. Sizes and constants are
@@ -70,23 +79,39 @@ def scaled_rope_frequencies(rot: dict):
 
 
 class LatentAttention(nn.Module):
+    """rot None (with rot_dim 0): no rotated key part, no positions.
+    q_rank: the queries come from a normed low-rank latent of that size
+    (the merged projection then holds the latent's rows instead of q).
+    gated False: no sigmoid output gate."""
+
     def __init__(self, width: int, heads: int, dim: int, rot_dim: int,
-                 vdim: int, kv_rank: int, scale: float, rot: dict,
-                 norm_eps: float, kv_from: Optional[int], dtype):
+                 vdim: int, kv_rank: int, scale: float, rot: Optional[dict],
+                 norm_eps: float, kv_from: Optional[int], dtype,
+                 q_rank: Optional[int] = None, gated: bool = True):
         super().__init__()
         self.heads, self.dim, self.rot_dim = heads, dim, rot_dim
         self.vdim, self.kv_rank = vdim, kv_rank
         self.scale, self.eps, self.kv_from = float(scale), norm_eps, kv_from
-        self.rot_dims = int(rot["dims"])
+        self.rot_dims = int(rot["dims"]) if rot else 0
         if self.rot_dims > rot_dim or self.rot_dims % 2:
             raise ValueError("rotary dims must be even and <= rot_dim")
-        inv_freq, self.mscale = scaled_rope_frequencies(rot)
+        if rot:
+            inv_freq, self.mscale = scaled_rope_frequencies(rot)
+        else:
+            inv_freq, self.mscale = torch.zeros(0, dtype=torch.float64), 1.0
         self.register_buffer("inv_freq", inv_freq, persistent=False)
+        self.q_rank, self.gated = q_rank, gated
         self.q_width = heads * (dim + rot_dim)
+        self.q_in = q_rank if q_rank else self.q_width
         self.dkv_width = 0 if kv_from is not None else kv_rank + rot_dim
-        self.g_width = heads * vdim
+        self.g_width = heads * vdim if gated else 0
         # merged-projection rows owned by this mixer: [q | dkv | g]
-        self.in_width = self.q_width + self.dkv_width + self.g_width
+        self.in_width = self.q_in + self.dkv_width + self.g_width
+        if q_rank:
+            self.dq_norm = nn.Parameter(torch.ones(q_rank,
+                                                   dtype=torch.float32))
+            self.w_uq = nn.Parameter(torch.empty(self.q_width, q_rank,
+                                                 dtype=dtype))
         if kv_from is None:
             self.dkv_norm = nn.Parameter(torch.ones(kv_rank,
                                                     dtype=torch.float32))
@@ -106,20 +131,29 @@ class LatentAttention(nn.Module):
     def forward(self, proj, positions, cache, meta: AttnMetadata, aux):
         T = proj.shape[0]
         H, dim, rd, r = self.heads, self.dim, self.rot_dim, self.kv_rank
-        q = proj[:, :self.q_width].unflatten(-1, (H, dim + rd))
-        hops.rope_interleaved_(q, positions, self.inv_freq, self.mscale, dim,
-                               self.rot_dims)
+        if self.q_rank:
+            cq = hops.group_rmsnorm(proj[:, :self.q_in], self.dq_norm,
+                                    self.eps, 1, proj.dtype)
+            q = F.linear(cq, self.w_uq).unflatten(-1, (H, dim + rd))
+        else:
+            q = proj[:, :self.q_width].unflatten(-1, (H, dim + rd))
+        if self.rot_dims:
+            hops.rope_interleaved_(q, positions, self.inv_freq, self.mscale,
+                                   dim, self.rot_dims)
         if self.kv_from is None:
-            dkv = proj[:, self.q_width:self.q_width + self.dkv_width]
+            dkv = proj[:, self.q_in:self.q_in + self.dkv_width]
             hops.latent_kv_store(dkv, self.dkv_norm, self.eps, positions,
                                  self.inv_freq, self.mscale, self.rot_dims,
                                  cache, meta.slot_mapping, r)
-        gate = proj[:, self.q_width + self.dkv_width:self.in_width]
         # fold the queries through the key up-projection: [H,T,dim]x[H,dim,r]
         q_abs = torch.bmm(q[..., :dim].transpose(0, 1), self.w_uk)
-        qf = torch.empty(T, H, r + rd, dtype=proj.dtype, device=proj.device)
-        qf[..., :r] = q_abs.transpose(0, 1)
-        qf[..., r:] = q[..., dim:]
+        if rd:
+            qf = torch.empty(T, H, r + rd, dtype=proj.dtype,
+                             device=proj.device)
+            qf[..., :r] = q_abs.transpose(0, 1)
+            qf[..., r:] = q[..., dim:]
+        else:
+            qf = q_abs.transpose(0, 1).contiguous()
         lat = torch.empty(T, H, r, dtype=torch.float32, device=proj.device)
         np_, nd = meta.num_prefill_tokens, meta.num_decode_tokens
         if np_:
@@ -132,6 +166,9 @@ class LatentAttention(nn.Module):
         # value up-projection per head: [H,T,r] x [H,r,vdim]
         o = torch.bmm(lat.to(proj.dtype).transpose(0, 1), self.w_uv_t)
         o = o.transpose(0, 1).reshape(T, H * self.vdim)
+        if not self.gated:
+            return F.linear(o, self.o_proj)
+        gate = proj[:, self.q_in + self.dkv_width:self.in_width]
         y = hops.norm_sigmoid_gate(o.float(), None, gate, self.eps, proj.dtype)
         return F.linear(y, self.o_proj)
 
@@ -375,3 +412,111 @@ class ParallelMixer(nn.Module):
         return (self.left(proj[:, :lw], positions, cache[0], meta, aux),
                 self.right(proj[:, lw:self.in_width], positions, cache[1],
                            meta, aux))
+
+
+class SinkWindowAttention(nn.Module):
+    """in_proj rows: [q: heads*dim | k: kv_heads*dim | v: kv_heads*vdim |
+    g: heads]. window 0 = every earlier key."""
+
+    def __init__(self, width: int, heads: int, kv_heads: int, dim: int,
+                 vdim: int, rot: Optional[dict], scale: float, window: int,
+                 norm_eps: float, dtype):
+        super().__init__()
+        if heads % kv_heads:
+            raise ValueError("heads must be a multiple of kv_heads")
+        self.heads, self.kv_heads, self.dim, self.vdim = heads, kv_heads, \
+            dim, vdim
+        self.scale, self.window, self.eps = float(scale), int(window), norm_eps
+        self.rot_dims = int(rot["dims"]) if rot else 0
+        if self.rot_dims > dim or self.rot_dims % 2:
+            raise ValueError("rotary dims must be even and <= dim")
+        if self.rot_dims:
+            inv_freq, _ = scaled_rope_frequencies(
+                dict(base=rot["base"], dims=rot["dims"]))
+        else:
+            inv_freq = torch.zeros(0, dtype=torch.float64)
+        self.register_buffer("inv_freq", inv_freq, persistent=False)
+        self.cq, self.ck, self.cv = heads * dim, kv_heads * dim, \
+            kv_heads * vdim
+        self.in_width = self.cq + self.ck + self.cv + heads
+        f32 = dict(dtype=torch.float32)
+        self.q_norm = nn.Parameter(torch.ones(self.cq, **f32))
+        self.k_norm = nn.Parameter(torch.ones(self.ck, **f32))
+        self.sink = nn.Parameter(torch.zeros(heads, **f32))
+        self.o_proj = nn.Parameter(torch.empty(width, heads * vdim,
+                                               dtype=dtype))
+
+    def cache_spec(self):
+        return PagedKV(self.kv_heads, self.dim, self.vdim)
+
+    def forward(self, proj, positions, cache, meta: AttnMetadata, aux):
+        k_cache, v_cache = cache
+        T, cq, ck, cv = proj.shape[0], self.cq, self.ck, self.cv
+        H = self.heads
+        q = hops.rownorm_rope_store(
+            proj[:, :cq], proj[:, cq:cq + ck], proj[:, cq + ck:cq + ck + cv],
+            self.q_norm, self.k_norm, self.eps, positions, self.inv_freq,
+            self.rot_dims, H, self.kv_heads, k_cache, v_cache,
+            meta.slot_mapping)
+        gate = proj[:, cq + ck + cv:self.in_width]
+        o = torch.empty(T, H, self.vdim, dtype=torch.float32,
+                        device=proj.device)
+        for rows, cu_q, _, _, seq_lens, tables, _ in _halves(meta, aux):
+            hops.capped_attn(q[rows], k_cache, v_cache, tables, cu_q,
+                             seq_lens, H, self.scale, 0.0, o[rows],
+                             window=self.window, sink=self.sink)
+        y = hops.norm_sigmoid_gate(o.view(T, H * self.vdim), None, gate, 0.0,
+                                   proj.dtype, gate_cols=self.vdim)
+        return F.linear(y, self.o_proj)
+
+
+class GatedDeltaRule(nn.Module):
+    """in_proj rows: [q: kv_heads*dim | k: kv_heads*dim | v: heads*vdim |
+    g: heads*vdim | b: heads | a: heads]; q, k, v pass the short
+    convolution (filters stacked in that order) and SiLU."""
+
+    def __init__(self, width: int, heads: int, kv_heads: int, dim: int,
+                 vdim: int, taps: int, norm_eps: float, dtype):
+        super().__init__()
+        if heads % kv_heads:
+            raise ValueError("heads must be a multiple of kv_heads")
+        self.heads, self.kv_heads, self.dim, self.vdim = heads, kv_heads, \
+            dim, vdim
+        self.taps, self.eps = taps, norm_eps
+        self.qk_width, self.v_width = kv_heads * dim, heads * vdim
+        self.conv_ch = 2 * self.qk_width + self.v_width
+        self.in_width = self.conv_ch + self.v_width + 2 * heads
+        f32 = dict(dtype=torch.float32)
+        self.conv_w = nn.Parameter(torch.empty(self.conv_ch, taps, dtype=dtype))
+        self.dt_bias = nn.Parameter(torch.zeros(heads, **f32))
+        self.A_log = nn.Parameter(torch.zeros(heads, **f32))
+        self.out_norm = nn.Parameter(torch.ones(vdim, **f32))
+        self.o_proj = nn.Parameter(torch.empty(width, self.v_width,
+                                               dtype=dtype))
+
+    def cache_spec(self):
+        return CacheGroup((ConvState(self.conv_ch, self.taps),
+                           RecurrentState(self.heads, self.dim, self.vdim)))
+
+    def forward(self, proj, positions, cache, meta: AttnMetadata, aux):
+        conv_state, state = cache
+        T, a, b, H = proj.shape[0], self.qk_width, self.v_width, self.heads
+        c = self.conv_ch
+        u_all = proj[:, :c]
+        gate = proj[:, c:c + b]
+        beta, dt = proj[:, c + b:c + b + H], proj[:, c + b + H:self.in_width]
+        o = torch.empty(T, H, self.vdim, dtype=torch.float32,
+                        device=proj.device)
+        for rows, cu_q, ctx, slots, _, _, max_len in _halves(meta, aux):
+            u = u_all[rows]
+            x = hops.short_conv(u, self.conv_w, None, conv_state, 0, slots,
+                                cu_q, ctx, 1, c, act_silu=True)
+            hops.short_conv_state_(conv_state, u, slots, cu_q)
+            hops.delta_rule(x[:, :a], x[:, a:2 * a], x[:, 2 * a:], beta[rows],
+                            dt[rows], self.dt_bias, self.A_log, state, slots,
+                            cu_q, ctx, self.kv_heads, o[rows],
+                            max_q_len=max_len)
+        y = hops.gated_group_norm(o.view(T, b), self.out_norm, gate, self.eps,
+                                  H, act_silu=True, gate_first=False,
+                                  out_dtype=proj.dtype)
+        return F.linear(y, self.o_proj)

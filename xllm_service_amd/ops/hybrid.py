@@ -54,13 +54,15 @@ def gated_norm_residual(res, y, gate, gate_bias, w, ls, mult: float,
 
 
 def norm_sigmoid_gate(o, w: Optional[torch.Tensor], gate, eps: float,
-                      out_dtype):
-    """(rmsnorm(o) * w if w is given else o) * sigmoid(gate); o fp32 2-D."""
+                      out_dtype, gate_cols: int = 1):
+    """(rmsnorm(o) * w if w is given else o) * sigmoid(gate); o fp32 2-D.
+    gate_cols > 1: gate has o's width / gate_cols entries per row, each
+    serving that many neighbouring columns (one gate per head)."""
     if o.is_cuda:
         out = torch.empty(o.shape, dtype=out_dtype, device=o.device)
-        _hyb().norm_sigmoid_gate(out, o, w, gate, eps)
+        _hyb().norm_sigmoid_gate(out, o, w, gate, eps, gate_cols)
         return out
-    return ref.norm_sigmoid_gate(o, w, gate, eps, out_dtype)
+    return ref.norm_sigmoid_gate(o, w, gate, eps, out_dtype, gate_cols)
 
 
 def silu_mul(x):
@@ -264,12 +266,67 @@ def gated_group_norm(o, w, gate, eps: float, groups: int, *, act_silu: bool,
 
 
 def capped_attn(q, k_cache, v_cache, block_tables, cu_q, seq_lens,
-                heads: int, scale: float, cap: float, out):
-    """out fp32 [T, heads, Dv] (written). cu_q None: decode rows."""
+                heads: int, scale: float, cap: float, out, window: int = 0,
+                sink: Optional[torch.Tensor] = None):
+    """out fp32 [T, heads, Dv] (written). cu_q None: decode rows. window > 0
+    limits a query to the last `window` keys (itself included); sink fp32
+    [heads] adds exp(sink_h) to the softmax denominator."""
     if q.is_cuda:
         _hyb().capped_attn(out, q, k_cache, v_cache, block_tables, cu_q,
-                           seq_lens, heads, scale, cap)
+                           seq_lens, heads, scale, cap, window, sink)
         return out
     out.copy_(ref.capped_attn(q, k_cache, v_cache, block_tables, cu_q,
-                              seq_lens, heads, scale, cap))
+                              seq_lens, heads, scale, cap, window, sink))
     return out
+
+
+# ---- post-norm residual, whole-row q/k norm, delta rule, GELU gate ----------
+def norm_residual_add_(x, y, w1, eps: float, out_dtype):
+    """x (fp32 [T, W], in place) += y / rms(y) * w1; returns the new x in
+    out_dtype (what the next sublayer multiplies)."""
+    if x.is_cuda:
+        h = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+        _hyb().norm_residual_add(x, h, y, w1, eps)
+        return h
+    return ref.norm_residual_add(x, y, w1, eps, out_dtype)
+
+
+def rownorm_rope_store(q, k, v, q_w, k_w, eps: float, positions, inv_freq,
+                       rot_dims: int, heads: int, kv_heads: int, k_cache,
+                       v_cache, slot_mapping):
+    """RMS norm of the whole q row [T, heads*D] and k row [T, kv_heads*D]
+    (weights q_w, k_w), rotate-half positions on the first rot_dims entries
+    of every head. Returns the new q as a contiguous tensor; k and v go
+    into the paged caches at the tokens' slots."""
+    if q.is_cuda:
+        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+        _hyb().rownorm_rope_store(out, q, k, v, q_w, k_w, eps, positions,
+                                  inv_freq, rot_dims, heads, kv_heads,
+                                  k_cache, v_cache, slot_mapping)
+        return out
+    return ref.rownorm_rope_store(q, k, v, q_w, k_w, eps, positions,
+                                  inv_freq, rot_dims, heads, kv_heads,
+                                  k_cache, v_cache, slot_mapping)
+
+
+def delta_rule(q, k, v, b, a, dt_bias, A_log, state, slots, cu_q, ctx_lens,
+               groups: int, out, max_q_len: int = 0):
+    """out fp32 [T, H, Dv] (written); see ref.delta_rule. q/k/v/b/a are row
+    views of the projections; state fp32 [slots, H, D, Dv] in place."""
+    if q.is_cuda:
+        _hyb().delta_rule(out, q, k, v, b, a, dt_bias, A_log, state, slots,
+                          cu_q, ctx_lens, groups)
+        return out
+    out.copy_(ref.delta_rule(q, k, v, b, a, dt_bias, A_log, state, slots,
+                             cu_q, ctx_lens, groups))
+    return out
+
+
+def gelu_tanh_mul(x):
+    """[..., 2F] -> gelu_tanh(x[..., :F]) * x[..., F:]."""
+    if x.is_cuda:
+        out = torch.empty(x.shape[:-1] + (x.shape[-1] // 2,), dtype=x.dtype,
+                          device=x.device)
+        _hyb().gelu_tanh_mul(out, x)
+        return out
+    return ref.gelu_tanh_mul(x)

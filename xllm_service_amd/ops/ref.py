@@ -187,12 +187,16 @@ def gated_norm_residual(res, y, gate, gate_bias, w, ls, mult, eps, groups):
     return res
 
 
-def norm_sigmoid_gate(o, w, gate, eps, out_dtype):
-    """rmsnorm(o) * w * sigmoid(gate); w None skips the norm."""
+def norm_sigmoid_gate(o, w, gate, eps, out_dtype, gate_cols=1):
+    """rmsnorm(o) * w * sigmoid(gate); w None skips the norm. gate_cols > 1:
+    one gate entry serves that many neighbouring columns of o."""
     z = o.float()
     if w is not None:
         z = z * torch.rsqrt(z.pow(2).mean(-1, keepdim=True) + eps) * w.float()
-    return (z * torch.sigmoid(gate.float())).to(out_dtype)
+    g = torch.sigmoid(gate.float())
+    if gate_cols > 1:
+        g = g.repeat_interleave(gate_cols, -1)
+    return (z * g).to(out_dtype)
 
 
 def rope_interleaved(x, positions, inv_freq, mscale, rot_dims):
@@ -449,10 +453,12 @@ def store_paged(x, cache, slot_mapping):
 
 
 def capped_attn(q, k_cache, v_cache, block_tables, cu_q, seq_lens, heads,
-                scale, cap):
+                scale, cap, window=0, sink=None):
     """Causal softmax attention of q [T, heads*D] over the paged caches
     [blocks, n_kv, block, D|Dv]; scores scale * q.k, then cap * tanh(. /
-    cap) when cap > 0. Returns fp32 [T, heads, Dv]."""
+    cap) when cap > 0. window > 0: position i sees only the keys j with
+    i - j < window. sink [heads]: exp(sink_h) joins the softmax denominator
+    (a key without a value). Returns fp32 [T, heads, Dv]."""
     T = q.shape[0]
     nb, n_kv, bs, D = k_cache.shape
     Dv = v_cache.shape[3]
@@ -474,7 +480,104 @@ def capped_attn(q, k_cache, v_cache, block_tables, cu_q, seq_lens, heads,
         sc = torch.einsum("thd,hld->thl", qq, kk) * scale
         if cap and cap > 0:
             sc = cap * torch.tanh(sc / cap)
-        mask = torch.arange(L)[None, :] > (ctx + torch.arange(q1 - q0))[:, None]
+        qpos = (ctx + torch.arange(q1 - q0))[:, None]
+        mask = torch.arange(L)[None, :] > qpos
+        if window and window > 0:
+            mask = mask | (torch.arange(L)[None, :] <= qpos - window)
         sc = sc.masked_fill(mask[:, None, :], float("-inf"))
-        out[q0:q1] = torch.einsum("thl,hlv->thv", torch.softmax(sc, -1), vv)
+        if sink is None:
+            p = torch.softmax(sc, -1)
+        else:
+            sk = sink.float()[None, :, None]
+            m = torch.maximum(sc.max(-1, keepdim=True).values, sk)
+            e = torch.exp(sc - m)
+            p = e / (e.sum(-1, keepdim=True) + torch.exp(sk - m))
+        out[q0:q1] = torch.einsum("thl,hlv->thv", p, vv)
     return out
+
+
+# ---------------------------------------------------------------------------
+# Post-norm residual, whole-row query/key norm with rotate-half positions,
+# gated delta rule, GELU-gated feed-forward. fp32 throughout.
+# ---------------------------------------------------------------------------
+def norm_residual_add(x, y, w1, eps, out_dtype):
+    """x (fp32, in place) += y / rms(y) * w1; returns x in out_dtype."""
+    yf = y.float()
+    x.add_(yf * torch.rsqrt(yf.pow(2).mean(-1, keepdim=True) + eps) * w1)
+    return x.to(out_dtype)
+
+
+def rope_halves(x, positions, inv_freq, rot_dims):
+    """Entry i < rot_dims/2 of the last dim of x [T, H, D] turns together
+    with entry i + rot_dims/2 by pos * inv_freq[i] (fp64 angles)."""
+    if not rot_dims:
+        return x.float()
+    half = rot_dims // 2
+    a = positions.double()[:, None] * inv_freq.double()[None, :]
+    cos, sin = torch.cos(a).float()[:, None, :], torch.sin(a).float()[:, None, :]
+    xf = x.float()
+    u, v = xf[..., :half], xf[..., half:rot_dims]
+    return torch.cat([u * cos - v * sin, v * cos + u * sin,
+                      xf[..., rot_dims:]], -1)
+
+
+def rownorm_rope_store(q, k, v, q_w, k_w, eps, positions, inv_freq, rot_dims,
+                       heads, kv_heads, k_cache, v_cache, slot_mapping):
+    """q [T, heads*D] and k [T, kv_heads*D]: RMS norm over the whole row
+    times q_w / k_w, then the rotate-half turn per head. Returns the new
+    q; k and v [T, kv_heads*Dv] go to the paged caches."""
+    T = q.shape[0]
+
+    def norm(z, w):
+        zf = z.float()
+        return zf * torch.rsqrt(zf.pow(2).mean(-1, keepdim=True) + eps) * w
+    qn = rope_halves(norm(q, q_w).view(T, heads, -1), positions, inv_freq,
+                     rot_dims)
+    kn = rope_halves(norm(k, k_w).view(T, kv_heads, -1), positions, inv_freq,
+                     rot_dims)
+    store_paged(kn.reshape(T, -1).to(k.dtype), k_cache, slot_mapping)
+    store_paged(v, v_cache, slot_mapping)
+    return qn.reshape(T, -1).to(q.dtype)
+
+
+def delta_rule(q, k, v, b, a, dt_bias, A_log, state, slots, cu_q, ctx_lens,
+               groups):
+    """Gated delta rule. Per head, with unit k and q (q also times
+    D^-1/2), beta = sigmoid(b), g = exp(-exp(A_log) softplus(a + dt_bias)):
+    S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q. q/k
+    [T, groups*D] shared by the heads of a group; state fp32
+    [slots, H, D, Dv]; returns fp32 [T, H, Dv]."""
+    H, D, Dv = state.shape[1:]
+    T = q.shape[0]
+    per = H // groups
+
+    def unit(z):
+        zf = z.float().view(T, groups, D)
+        zf = zf * torch.rsqrt(zf.pow(2).sum(-1, keepdim=True) + 1e-6)
+        return zf.repeat_interleave(per, 1)
+    qf, kf = unit(q) * D ** -0.5, unit(k)
+    vf = v.float().view(T, H, Dv)
+    beta = torch.sigmoid(b.float())
+    g = torch.exp(-torch.exp(A_log) * torch.nn.functional.softplus(
+        a.float() + dt_bias, threshold=30.0))
+    out = torch.zeros(T, H, Dv, dtype=torch.float32)
+    for s, t0, t1 in _seq_ranges(T, slots, cu_q):
+        slot = int(slots[s])
+        if slot >= 0 and int(ctx_lens[s]) > 0:
+            S = state[slot].clone()
+        else:
+            S = torch.zeros(H, D, Dv, dtype=torch.float32)
+        for t in range(t0, t1):
+            S = g[t][:, None, None] * S
+            u = beta[t][:, None] * (vf[t] - torch.einsum("hdv,hd->hv", S,
+                                                         kf[t]))
+            S = S + kf[t][:, :, None] * u[:, None, :]
+            out[t] = torch.einsum("hdv,hd->hv", S, qf[t])
+        if slot >= 0:
+            state[slot] = S
+    return out
+
+
+def gelu_tanh_mul(x):
+    """[..., 2F] -> gelu_tanh(x[..., :F]) * x[..., F:], dtype preserved."""
+    return gelu_and_mul(x)
