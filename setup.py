@@ -47,8 +47,9 @@ ext_modules = [
         },
     ),
     # hybrid sequence mixers (latent attention, decayed and gated linear
-    # recurrences, soft-capped paged attention, short convolutions), grouped
-    # norms, residual streams and routed experts; bf16 and fp32 activations
+    # recurrences, the gated delta rule, soft-capped / windowed paged attention,
+    # short convolutions), grouped and post norms, residual streams and routed
+    # experts; bf16 and fp32 activations
     CUDAExtension(
         name="xllm_service_amd._ops_hybrid",
         sources=[
@@ -57,7 +58,8 @@ ext_modules = [
                       "latent_attn_mfma.hip", "decay_attn.hip", "moe.hip",
                       "streams.hip", "short_conv.hip",
                       "gated_recurrence.hip", "capped_attn.hip",
-                      "capped_attn_mfma.hip")
+                      "capped_attn_mfma.hip", "rownorm_rope.hip",
+                      "delta_rule.hip")
         ],
         extra_compile_args={
             "cxx": ["-O3", "-std=c++17"],

@@ -21,9 +21,25 @@ void launch_gated_norm_residual(float*, const TY*, const TG*, const float*,
                                 int, int, long, hipStream_t);
 template <typename T>
 void launch_norm_sigmoid_gate(T*, const float*, const float*, const T*, float,
-                              int, int, long, hipStream_t);
+                              int, int, long, int, hipStream_t);
+template <typename T>
+void launch_norm_residual_add(float*, T*, const T*, const float*, float, int,
+                              int, long, hipStream_t);
 template <typename T>
 void launch_silu_mul(T*, const T*, long, int, hipStream_t);
+template <typename T>
+void launch_gelu_tanh_mul(T*, const T*, long, int, hipStream_t);
+template <typename T>
+void launch_rownorm_rope_store(T*, const T*, const T*, const T*, long, long,
+                               long, const float*, const float*, float,
+                               const long*, const double*, int, int, int, int,
+                               int, int, T*, T*, const long*, int,
+                               hipStream_t);
+template <typename T>
+void launch_delta_rule(float*, const T*, const T*, const T*, const T*,
+                       const T*, long, long, long, long, long, const float*,
+                       const float*, float*, const int*, const int*,
+                       const int*, int, int, int, int, int, hipStream_t);
 template <typename T>
 void launch_rope_interleaved(T*, const long*, const double*, float, int, int,
                              int, long, long, int, hipStream_t);
@@ -88,11 +104,12 @@ void launch_capped_attn_mfma(float*, float*, float*, const unsigned short*,
                              const unsigned short*, const unsigned short*,
                              const int*, const int*, const int*, int, int, int,
                              int, int, int, int, int, float, float, long, int,
-                             hipStream_t);
+                             int, const float*, hipStream_t);
 template <typename T>
 void launch_capped_attn(float*, const T*, const T*, const T*, const int*,
                         const int*, const int*, int, int, int, int, int, int,
-                        int, int, float, float, long, hipStream_t);
+                        int, int, float, float, long, int, const float*,
+                        hipStream_t);
 }  // namespace hyb
 }  // namespace xllm
 
@@ -172,12 +189,13 @@ void gated_norm_residual(Tensor res, Tensor y, Tensor gate,
 }
 
 void norm_sigmoid_gate(Tensor out, Tensor o, c10::optional<Tensor> w,
-                       Tensor gate, double eps) {
+                       Tensor gate, double eps, long gate_cols) {
   CHK_ACT(out); CHK_F32C(o); CHK_ACT(gate);
   TORCH_CHECK(out.is_contiguous() && out.dim() == 2 && gate.dim() == 2);
   const int rows = out.size(0), n = out.size(1);
+  TORCH_CHECK(gate_cols >= 1 && n % gate_cols == 0);
   TORCH_CHECK(o.numel() == (long)rows * n && gate.size(0) == rows &&
-              gate.size(1) == n && gate.dtype() == out.dtype());
+              gate.size(1) == n / gate_cols && gate.dtype() == out.dtype());
   const float* wp = nullptr;
   if (w.has_value()) {
     CHK_F32C(*w);
@@ -185,9 +203,107 @@ void norm_sigmoid_gate(Tensor out, Tensor o, c10::optional<Tensor> w,
     wp = ptr<float>(*w);
   }
   if (is_f32(out))
-    hy::launch_norm_sigmoid_gate<float>(ptr<float>(out), ptr<float>(o), wp, ptr<float>(gate), eps, rows, n, gate.stride(0), cur());
+    hy::launch_norm_sigmoid_gate<float>(ptr<float>(out), ptr<float>(o), wp, ptr<float>(gate), eps, rows, n, gate.stride(0), gate_cols, cur());
   else
-    hy::launch_norm_sigmoid_gate<bf>(ptr<bf>(out), ptr<float>(o), wp, ptr<bf>(gate), eps, rows, n, gate.stride(0), cur());
+    hy::launch_norm_sigmoid_gate<bf>(ptr<bf>(out), ptr<float>(o), wp, ptr<bf>(gate), eps, rows, n, gate.stride(0), gate_cols, cur());
+}
+
+// res fp32 [rows, width] += y / rms(y) * w1; h = the new res in y's type
+void norm_residual_add(Tensor res, Tensor h, Tensor y, Tensor w1, double eps) {
+  CHK_F32C(res); CHK_ACT(h); CHK_ACT(y); CHK_F32C(w1);
+  TORCH_CHECK(res.dim() == 2 && y.dim() == 2 && h.is_contiguous() &&
+              h.dtype() == y.dtype());
+  const int rows = res.size(0), width = res.size(1);
+  TORCH_CHECK(y.size(0) == rows && y.size(1) == width &&
+              h.numel() == res.numel() && w1.numel() == width);
+  if (is_f32(y))
+    hy::launch_norm_residual_add<float>(ptr<float>(res), ptr<float>(h), ptr<float>(y), ptr<float>(w1), eps, rows, width, y.stride(0), cur());
+  else
+    hy::launch_norm_residual_add<bf>(ptr<float>(res), ptr<bf>(h), ptr<bf>(y), ptr<float>(w1), eps, rows, width, y.stride(0), cur());
+}
+
+void gelu_tanh_mul(Tensor out, Tensor x) {
+  CHK_ACT(out); CHK_ACT(x);
+  TORCH_CHECK(out.is_contiguous() && x.is_contiguous() &&
+              out.dtype() == x.dtype());
+  const int F = out.size(-1);
+  TORCH_CHECK(x.size(-1) == 2 * F && x.numel() == 2 * out.numel());
+  const long rows = out.numel() / F;
+  if (is_f32(x)) hy::launch_gelu_tanh_mul<float>(ptr<float>(out), ptr<float>(x), rows, F, cur());
+  else hy::launch_gelu_tanh_mul<bf>(ptr<bf>(out), ptr<bf>(x), rows, F, cur());
+}
+
+// q_out [T, H*D] contiguous; q/k/v row views of a projection; caches
+// [blocks, n_kv, block, D | Dv]
+void rownorm_rope_store(Tensor q_out, Tensor q, Tensor k, Tensor v, Tensor wq,
+                        Tensor wk, double eps, Tensor pos, Tensor inv_freq,
+                        long rot, long heads, long n_kv, Tensor k_cache,
+                        Tensor v_cache, Tensor slot_mapping) {
+  CHK_ACT(q_out); CHK_ACT(q); CHK_ACT(k); CHK_ACT(v); CHK_F32C(wq);
+  CHK_F32C(wk); CHK_I64C(pos); CHK_I64C(slot_mapping); CHK_ACT(k_cache);
+  CHK_ACT(v_cache);
+  TORCH_CHECK(q.dim() == 2 && k.dim() == 2 && v.dim() == 2 &&
+              q_out.is_contiguous() && k_cache.dim() == 4 &&
+              v_cache.dim() == 4 && k_cache.is_contiguous() &&
+              v_cache.is_contiguous());
+  TORCH_CHECK(q.dtype() == k.dtype() && q.dtype() == v.dtype() &&
+              q.dtype() == q_out.dtype() && q.dtype() == k_cache.dtype() &&
+              q.dtype() == v_cache.dtype());
+  const int T = q.size(0), D = k_cache.size(3), Dv = v_cache.size(3);
+  const int bs = k_cache.size(2);
+  TORCH_CHECK(heads >= 1 && n_kv >= 1 && q.size(1) == heads * D &&
+              k.size(1) == n_kv * D && v.size(1) == n_kv * Dv &&
+              k.size(0) == T && v.size(0) == T && q_out.numel() == q.numel() &&
+              k_cache.size(1) == n_kv && v_cache.size(1) == n_kv &&
+              v_cache.size(2) == bs && v_cache.size(0) == k_cache.size(0) &&
+              wq.numel() == heads * D && wk.numel() == n_kv * D &&
+              pos.numel() == T && slot_mapping.numel() == T,
+              "rownorm_rope_store: bad shapes");
+  TORCH_CHECK(rot >= 0 && rot % 2 == 0 && rot <= D && rot <= 8192 &&
+              inv_freq.is_cuda() && inv_freq.dtype() == torch::kDouble &&
+              inv_freq.is_contiguous() && inv_freq.numel() == rot / 2);
+  if (is_f32(q))
+    hy::launch_rownorm_rope_store<float>(ptr<float>(q_out), ptr<float>(q), ptr<float>(k), ptr<float>(v), q.stride(0), k.stride(0), v.stride(0), ptr<float>(wq), ptr<float>(wk), eps, ptr<long>(pos), ptr<double>(inv_freq), rot, T, heads, n_kv, D, Dv, ptr<float>(k_cache), ptr<float>(v_cache), ptr<long>(slot_mapping), bs, cur());
+  else
+    hy::launch_rownorm_rope_store<bf>(ptr<bf>(q_out), ptr<bf>(q), ptr<bf>(k), ptr<bf>(v), q.stride(0), k.stride(0), v.stride(0), ptr<float>(wq), ptr<float>(wk), eps, ptr<long>(pos), ptr<double>(inv_freq), rot, T, heads, n_kv, D, Dv, ptr<bf>(k_cache), ptr<bf>(v_cache), ptr<long>(slot_mapping), bs, cur());
+}
+
+// out fp32 [T, H, Dv]; state fp32 [slots, H, D, Dv]; q/k [T, groups*D],
+// v [T, H*Dv], b/a [T, H] row views (after convolution: q, k, v)
+void delta_rule(Tensor out, Tensor q, Tensor k, Tensor v, Tensor b, Tensor a,
+                Tensor dt_bias, Tensor A_log, Tensor state, Tensor slots,
+                c10::optional<Tensor> cu_q, Tensor ctx_lens, long groups) {
+  CHK_F32C(out); CHK_ACT(q); CHK_ACT(k); CHK_ACT(v); CHK_ACT(b); CHK_ACT(a);
+  CHK_F32C(dt_bias); CHK_F32C(A_log); CHK_F32C(state); CHK_I32C(slots);
+  CHK_I32C(ctx_lens);
+  TORCH_CHECK(state.dim() == 4 && q.dim() == 2 && k.dim() == 2 &&
+              v.dim() == 2 && b.dim() == 2 && a.dim() == 2 &&
+              q.dtype() == k.dtype() && q.dtype() == v.dtype() &&
+              q.dtype() == b.dtype() && q.dtype() == a.dtype());
+  const int H = state.size(1), D = state.size(2), Dv = state.size(3);
+  const int T = q.size(0);
+  TORCH_CHECK(groups >= 1 && H % groups == 0 && q.size(1) == groups * D &&
+              k.size(1) == groups * D && v.size(1) == H * Dv &&
+              b.size(1) == H && a.size(1) == H && k.size(0) == T &&
+              v.size(0) == T && b.size(0) == T && a.size(0) == T &&
+              dt_bias.numel() == H && A_log.numel() == H,
+              "delta_rule: bad shapes");
+  TORCH_CHECK(D <= 256, "key dim > 256 unsupported");
+  TORCH_CHECK(out.numel() == (long)T * H * Dv);
+  const int n_seqs = slots.numel();
+  TORCH_CHECK(ctx_lens.numel() == n_seqs);
+  const int* cu = nullptr;
+  if (cu_q.has_value()) {
+    CHK_I32C(*cu_q);
+    TORCH_CHECK(cu_q->numel() == n_seqs + 1);
+    cu = ptr<int>(*cu_q);
+  } else {
+    TORCH_CHECK(n_seqs == T, "decode: one sequence per token");
+  }
+  if (is_f32(q))
+    hy::launch_delta_rule<float>(ptr<float>(out), ptr<float>(q), ptr<float>(k), ptr<float>(v), ptr<float>(b), ptr<float>(a), q.stride(0), k.stride(0), v.stride(0), b.stride(0), a.stride(0), ptr<float>(dt_bias), ptr<float>(A_log), ptr<float>(state), ptr<int>(slots), cu, ptr<int>(ctx_lens), n_seqs, H, groups, D, Dv, cur());
+  else
+    hy::launch_delta_rule<bf>(ptr<float>(out), ptr<bf>(q), ptr<bf>(k), ptr<bf>(v), ptr<bf>(b), ptr<bf>(a), q.stride(0), k.stride(0), v.stride(0), b.stride(0), a.stride(0), ptr<float>(dt_bias), ptr<float>(A_log), ptr<float>(state), ptr<int>(slots), cu, ptr<int>(ctx_lens), n_seqs, H, groups, D, Dv, cur());
 }
 
 void silu_mul(Tensor out, Tensor x) {
@@ -677,7 +793,8 @@ void gated_group_norm(Tensor out, Tensor o, Tensor w, Tensor gate, double eps,
 // out fp32 [T, H, Dv]; q [T, H*D] row view; caches [blocks, n_kv, bs, D|Dv]
 void capped_attn(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
                  Tensor block_tables, c10::optional<Tensor> cu_q,
-                 Tensor seq_lens, long heads, double scale, double cap) {
+                 Tensor seq_lens, long heads, double scale, double cap,
+                 long window, c10::optional<Tensor> sink) {
   CHK_F32C(out); CHK_ACT(q); CHK_ACT(k_cache); CHK_ACT(v_cache);
   CHK_I32C(block_tables); CHK_I32C(seq_lens);
   TORCH_CHECK(q.dim() == 2 && k_cache.dim() == 4 && v_cache.dim() == 4 &&
@@ -701,6 +818,13 @@ void capped_attn(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
   } else {
     TORCH_CHECK(n_seqs == T, "decode: one sequence per token");
   }
+  TORCH_CHECK(window >= 0 && window < (1L << 30), "bad window");
+  const float* sinkp = nullptr;
+  if (sink.has_value()) {
+    CHK_F32C(*sink);
+    TORCH_CHECK(sink->numel() == heads);
+    sinkp = ptr<float>(*sink);
+  }
   // bf16: MFMA kernel when the sizes fit one of its instantiations
   if (is_bf16(q) && hy::capped_attn_mfma_class(D, Dv) != 0 &&
       q.stride(0) % 8 == 0 &&
@@ -715,7 +839,8 @@ void capped_attn(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
       const int per = heads / n_kv;
       const int rows_wg = per <= 16 ? 16 : per <= 32 ? 32 : 64;
       const long wgs = (long)T * n_kv * ((per + rows_wg - 1) / rows_wg);
-      const long max_tiles = ((long)block_tables.size(1) * bs + 31) / 32;
+      long max_tiles = ((long)block_tables.size(1) * bs + 31) / 32;
+      if (window > 0) max_tiles = std::min<long>(max_tiles, (window + 31) / 32 + 1);
       n_part = (int)std::min<long>(std::min<long>(32, (max_tiles + 1) / 2),
                                    std::max<long>(1, 1024 / wgs));
       n_part = std::max(n_part, 1);
@@ -732,14 +857,14 @@ void capped_attn(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
         n_part > 1 ? ptr<float>(ws_ml) : nullptr, ptr<bf>(q), ptr<bf>(k_cache),
         ptr<bf>(v_cache), ptr<int>(block_tables), cu, ptr<int>(seq_lens), T,
         n_seqs, heads, n_kv, D, Dv, bs, block_tables.size(1), scale, cap,
-        q.stride(0), n_part, cur());
+        q.stride(0), n_part, window, sinkp, cur());
     return;
   }
   TORCH_CHECK((size_t)4 * D * 4 <= 64 * 1024, "query row too wide for LDS");
   if (is_f32(q))
-    hy::launch_capped_attn<float>(ptr<float>(out), ptr<float>(q), ptr<float>(k_cache), ptr<float>(v_cache), ptr<int>(block_tables), cu, ptr<int>(seq_lens), T, n_seqs, heads, n_kv, D, Dv, bs, block_tables.size(1), scale, cap, q.stride(0), cur());
+    hy::launch_capped_attn<float>(ptr<float>(out), ptr<float>(q), ptr<float>(k_cache), ptr<float>(v_cache), ptr<int>(block_tables), cu, ptr<int>(seq_lens), T, n_seqs, heads, n_kv, D, Dv, bs, block_tables.size(1), scale, cap, q.stride(0), window, sinkp, cur());
   else
-    hy::launch_capped_attn<bf>(ptr<float>(out), ptr<bf>(q), ptr<bf>(k_cache), ptr<bf>(v_cache), ptr<int>(block_tables), cu, ptr<int>(seq_lens), T, n_seqs, heads, n_kv, D, Dv, bs, block_tables.size(1), scale, cap, q.stride(0), cur());
+    hy::launch_capped_attn<bf>(ptr<float>(out), ptr<bf>(q), ptr<bf>(k_cache), ptr<bf>(v_cache), ptr<int>(block_tables), cu, ptr<int>(seq_lens), T, n_seqs, heads, n_kv, D, Dv, bs, block_tables.size(1), scale, cap, q.stride(0), window, sinkp, cur());
 }
 
 }  // namespace
@@ -765,4 +890,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("gated_recurrence", &gated_recurrence);
   m.def("gated_group_norm", &gated_group_norm);
   m.def("capped_attn", &capped_attn);
+  m.def("norm_residual_add", &norm_residual_add);
+  m.def("gelu_tanh_mul", &gelu_tanh_mul);
+  m.def("rownorm_rope_store", &rownorm_rope_store);
+  m.def("delta_rule", &delta_rule);
 }

@@ -5,6 +5,10 @@
 //   s_ij = scale * (q_i . k_j);  s_ij <- cap * tanh(s_ij / cap);
 //   o_i  = sum_j softmax_j(s_ij) v_j        over keys j <= i
 //
+// Optional: a sliding window (only the keys with i - j < window are seen) and
+// a per-head sink, a learned score without key or value whose exponential
+// joins the softmax denominator.
+//
 // Caches: keys [blocks, n_kv, block, D], values [blocks, n_kv, block, Dv].
 // Scores, softmax weights and the weighted sum are fp32 for both storage
 // types. One wavefront per (query token, head): 64 keys are scored per step,
@@ -26,7 +30,7 @@ __global__ void capped_attn_kernel(
     const int* __restrict__ block_tables, const int* __restrict__ cu_q,
     const int* __restrict__ seq_lens, int n_seqs, int heads, int n_kv, int D,
     int Dv, int block_size, int table_width, float scale, float cap,
-    long q_row_stride) {
+    long q_row_stride, int window, const float* __restrict__ sink) {
   extern __shared__ float smem[];
   const int t = blockIdx.x;
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
@@ -64,7 +68,8 @@ __global__ void capped_attn_kernel(
   for (int i = 0; i < CA_MAX_ACC; ++i) acc[i] = 0.f;
   const int n_acc = (Dv + 63) >> 6;
 
-  for (int k0 = 0; k0 < n_keys; k0 += 64) {
+  const int k_first = window > 0 ? max(0, n_keys - window) : 0;
+  for (int k0 = k_first; k0 < n_keys; k0 += 64) {
     const int key = k0 + lane;
     float sc = -INFINITY;
     if (key < n_keys) {
@@ -97,6 +102,14 @@ __global__ void capped_attn_kernel(
       }
     }
   }
+  if (sink != nullptr) {                  // a key without a value
+    const float sk = sink[h];
+    const float m_new = fmaxf(m, sk);
+    const float alpha = expf(m - m_new);
+    l = l * alpha + expf(sk - m_new);
+#pragma unroll
+    for (int i = 0; i < CA_MAX_ACC; ++i) acc[i] *= alpha;
+  }
   const float inv = (l > 0.f) ? 1.0f / l : 0.f;
   float* orow = out + ((long)t * heads + h) * Dv;
 #pragma unroll
@@ -112,7 +125,8 @@ void launch_capped_attn(float* out, const T* q, const T* k_cache,
                         const int* cu_q, const int* seq_lens, int tokens,
                         int n_seqs, int heads, int n_kv, int D, int Dv,
                         int block_size, int table_width, float scale,
-                        float cap, long q_row_stride, hipStream_t st) {
+                        float cap, long q_row_stride, int window,
+                        const float* sink, hipStream_t st) {
   if (tokens == 0) return;
   const int nw = heads < 4 ? heads : 4;
   dim3 grid(tokens, (heads + nw - 1) / nw);
@@ -120,14 +134,14 @@ void launch_capped_attn(float* out, const T* q, const T* k_cache,
                      (size_t)nw * D * sizeof(float), st, out, q, k_cache,
                      v_cache, block_tables, cu_q, seq_lens, n_seqs, heads,
                      n_kv, D, Dv, block_size, table_width, scale, cap,
-                     q_row_stride);
+                     q_row_stride, window, sink);
 }
 
 #define INST_CA(T)                                                          \
   template void launch_capped_attn<T>(                                      \
       float*, const T*, const T*, const T*, const int*, const int*,         \
       const int*, int, int, int, int, int, int, int, int, float, float,     \
-      long, hipStream_t);
+      long, int, const float*, hipStream_t);
 INST_CA(float)
 INST_CA(unsigned short)
 

@@ -33,6 +33,10 @@
 // Decode splits the context over `n_part` workgroups per (token, key/value
 // head); partial (acc, max, sum) triples are merged by a second small kernel.
 //
+// Sliding window: a row sees the keys [limit - window, limit); the tile loop
+// starts at the first tile any row of the workgroup needs. Sink: exp(sink_h)
+// joins the denominator once, at the end (or in the merge kernel).
+//
 // Fragment layouts of __builtin_amdgcn_mfma_f32_16x16x32_bf16 (lane l):
 //   A[l&15][(l>>4)*8 + j], B[(l>>4)*8 + j][l&15], C[(l>>4)*4 + r][l&15].
 #include "hybrid_common.h"
@@ -69,7 +73,7 @@ __global__ void __launch_bounds__(256) capped_attn_mfma_kernel(
     const int* __restrict__ block_tables, const int* __restrict__ cu_q,
     const int* __restrict__ seq_lens, int n_seqs, int heads, int n_kv, int D,
     int Dv, int block_size, int table_width, float scale, float cap,
-    long q_stride, int n_part) {
+    long q_stride, int n_part, int window, const float* __restrict__ sink) {
   extern __shared__ unsigned short cm_lds[];      // [key image | value image]
   __shared__ int tbl[512];                        // block ids of this key range
   constexpr int RT = 4 / CS;                      // row tiles per workgroup
@@ -110,8 +114,11 @@ __global__ void __launch_bounds__(256) capped_attn_mfma_kernel(
   const int last_row = min(row0 + ROWS_WG, rows_in_seq) - 1;
   const int kmax = ctx + last_row / per + 1;         // keys any row here sees
   const int n_tiles = (kmax + CM_KT - 1) / CM_KT;
-  const int tpp = (n_tiles + n_part - 1) / n_part;
-  const int t_begin = blockIdx.y * tpp;
+  // first key the earliest row of this workgroup sees
+  const int kmin = window > 0 ? max(0, ctx + row0 / per + 1 - window) : 0;
+  const int t_first = kmin / CM_KT;
+  const int tpp = (n_tiles - t_first + n_part - 1) / n_part;
+  const int t_begin = t_first + blockIdx.y * tpp;
   const int t_end = min(n_tiles, t_begin + tpp);
   const int* table = block_tables + (long)s * table_width;
 
@@ -121,6 +128,7 @@ __global__ void __launch_bounds__(256) capped_attn_mfma_kernel(
   const bool wave_on = row0 + rt * 16 < rows_in_seq;
   const bool row_ok = rho < rows_in_seq;
   const int limit = row_ok ? ctx + rho / per + 1 : 0;
+  const int lo = window > 0 ? max(0, limit - window) : 0;
   const int head = kvh * per + (row_ok ? rho % per : 0);
   const long tok = q0 + (row_ok ? rho / per : 0);
   const long grow = tok * heads + head;              // row in [T*H]
@@ -224,7 +232,7 @@ __global__ void __launch_bounds__(256) capped_attn_mfma_kernel(
         const int kk = k0 + g * 8 + h2 * 4 + rr;     // key of C row g*4+rr
         float sv = sacc[rr] * scale;
         if (cap > 0.f) sv = cap * cm_tanh(sv * inv_cap);
-        sc[h2 * 4 + rr] = (kk < limit) ? sv : -INFINITY;
+        sc[h2 * 4 + rr] = (kk < limit && kk >= lo) ? sv : -INFINITY;
       }
     }
     float mloc = sc[0];
@@ -296,6 +304,7 @@ __global__ void __launch_bounds__(256) capped_attn_mfma_kernel(
   }
   if (!wave_on || !row_ok) return;
   // acc[lb*4+nn][rr] = O^T[col = ((lb*CS+cpart)*4+nn)*16 + g*4 + rr][row n]
+  if (n_part == 1 && sink != nullptr) l += __expf(sink[head] - m);
   const float inv = l > 0.f ? 1.0f / l : 0.f;
   const long base = grow * n_part + blockIdx.y;
   float* orow = (n_part == 1) ? out + grow * Dv : ws_acc + base * Dv;
@@ -317,18 +326,21 @@ __global__ void __launch_bounds__(256) capped_attn_mfma_kernel(
 // out[row] = sum_p acc[row][p] e^(m_p - M) / sum_p l_p e^(m_p - M)
 __global__ void __launch_bounds__(256) capped_attn_merge_kernel(
     float* __restrict__ out, const float* __restrict__ ws_acc,
-    const float* __restrict__ ws_ml, int r, int n_part) {
+    const float* __restrict__ ws_ml, int r, int n_part, int heads,
+    const float* __restrict__ sink) {
   __shared__ float wgt[64];
-  const long row = blockIdx.x;
+  const long row = blockIdx.x;                 // token * heads + head
   const int tid = threadIdx.x;
   if (tid < 64) {
     const bool on = tid < n_part;
     const float mp = on ? ws_ml[(row * n_part + tid) * 2] : -INFINITY;
     const float lp = on ? ws_ml[(row * n_part + tid) * 2 + 1] : 0.f;
     float M = wave_reduce_max(mp);
+    const float sk = sink ? sink[row % heads] : -INFINITY;
+    M = fmaxf(M, sk);
     if (M == -INFINITY) M = 0.f;
     const float e = on ? __expf(mp - M) : 0.f;
-    const float L = wave_reduce_sum(lp * e);
+    const float L = wave_reduce_sum(lp * e) + (sink ? __expf(sk - M) : 0.f);
     wgt[tid] = (L > 0.f) ? e / L : 0.f;
   }
   __syncthreads();
@@ -359,8 +371,8 @@ void launch_capped_attn_mfma(float* out, float* ws_acc, float* ws_ml,
                              const int* seq_lens, int tokens, int n_seqs,
                              int heads, int n_kv, int D, int Dv,
                              int block_size, int table_width, float scale,
-                             float cap, long q_stride, int n_part,
-                             hipStream_t st) {
+                             float cap, long q_stride, int n_part, int window,
+                             const float* sink, hipStream_t st) {
   if (tokens == 0) return;
   const int cls = capped_attn_mfma_class(D, Dv);
   const int per = heads / n_kv;
@@ -378,7 +390,7 @@ void launch_capped_attn_mfma(float* out, float* ws_acc, float* ws_ml,
                      (size_t)(KQ * 2 + NO) * 1024, st, out, ws_acc, ws_ml,   \
                      q, k_cache, v_cache, block_tables, cu_q, seq_lens,      \
                      n_seqs, heads, n_kv, D, Dv, block_size, table_width,    \
-                     scale, cap, q_stride, n_part)
+                     scale, cap, q_stride, n_part, window, sink)
 #define CM_BY_CS(KQ, NO)                                                     \
   do {                                                                       \
     if (cs == 4) CM_LAUNCH(KQ, NO, 4);                                       \
@@ -394,7 +406,7 @@ void launch_capped_attn_mfma(float* out, float* ws_acc, float* ws_ml,
   if (n_part > 1)
     hipLaunchKernelGGL(capped_attn_merge_kernel,
                        dim3((unsigned)tokens * heads), dim3(256), 0, st, out,
-                       ws_acc, ws_ml, Dv, n_part);
+                       ws_acc, ws_ml, Dv, n_part, heads, sink);
 }
 
 }  // namespace hyb

@@ -66,13 +66,16 @@ __global__ void gated_norm_residual_kernel(
   }
 }
 
-// out = (w ? o / rms(o) * w : o) * sigmoid(gate);  o fp32 [rows, n]
+// out = (w ? o / rms(o) * w : o) * sigmoid(gate);  o fp32 [rows, n]; gate
+// entry i / gate_cols serves column i (gate_cols = head width: one gate
+// number per head)
 template <typename T>
 __global__ void norm_sigmoid_gate_kernel(T* __restrict__ out,
                                          const float* __restrict__ o,
                                          const float* __restrict__ w,
                                          const T* __restrict__ gate,
-                                         float eps, int n, long gate_stride) {
+                                         float eps, int n, long gate_stride,
+                                         int gate_cols) {
   __shared__ float tmp[16];
   const int row = blockIdx.x;
   const float* orow = o + (long)row * n;
@@ -86,7 +89,8 @@ __global__ void norm_sigmoid_gate_kernel(T* __restrict__ out,
   }
   for (int i = threadIdx.x; i < n; i += blockDim.x) {
     float v = orow[i] * rs * (w ? w[i] : 1.0f);
-    IO<T>::st(out + (long)row * n + i, v * sigmoidf_(IO<T>::ld(gr + i)));
+    IO<T>::st(out + (long)row * n + i,
+              v * sigmoidf_(IO<T>::ld(gr + i / gate_cols)));
   }
 }
 
@@ -131,10 +135,42 @@ __global__ void gated_group_norm_kernel(
   }
 }
 
-// out[r, i] = silu(x[r, i]) * x[r, F + i]
+// res[row] += y[row] / rms(y[row]) * w1, and the new residual row once more
+// in the activation type (the operand of the next sublayer's GEMM)
 template <typename T>
-__global__ void silu_mul_kernel(T* __restrict__ out, const T* __restrict__ x,
-                                long rows, int F) {
+__global__ void norm_residual_add_kernel(float* __restrict__ res,
+                                         T* __restrict__ h,
+                                         const T* __restrict__ y,
+                                         const float* __restrict__ w1,
+                                         float eps, int width, long y_stride) {
+  __shared__ float tmp[16];
+  const int row = blockIdx.x;
+  const T* yr = y + (long)row * y_stride;
+  float* rr = res + (long)row * width;
+  T* hr = h + (long)row * width;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    const float v = IO<T>::ld(yr + i);
+    ss += v * v;
+  }
+  ss = block_reduce_sum(ss, tmp);
+  const float rs = 1.0f / sqrtf(ss / (float)width + eps);
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    const float v = rr[i] + IO<T>::ld(yr + i) * rs * w1[i];
+    rr[i] = v;
+    IO<T>::st(hr + i, v);
+  }
+}
+
+XLLM_DEV float gelu_tanhf_(float z) {
+  return 0.5f * z *
+         (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+// out[r, i] = act(x[r, i]) * x[r, F + i]; GELU false: SiLU, true: tanh-GELU
+template <typename T, bool GELU>
+__global__ void act_mul_kernel(T* __restrict__ out, const T* __restrict__ x,
+                               long rows, int F) {
   const long n = rows * (long)F;
   for (long idx = blockIdx.x * (long)blockDim.x + threadIdx.x; idx < n;
        idx += (long)gridDim.x * blockDim.x) {
@@ -142,7 +178,7 @@ __global__ void silu_mul_kernel(T* __restrict__ out, const T* __restrict__ x,
     const int i = (int)(idx - r * F);
     const float g = IO<T>::ld(x + r * 2 * F + i);
     const float u = IO<T>::ld(x + r * 2 * F + F + i);
-    IO<T>::st(out + idx, siluf_(g) * u);
+    IO<T>::st(out + idx, (GELU ? gelu_tanhf_(g) : siluf_(g)) * u);
   }
 }
 
@@ -195,10 +231,19 @@ void launch_gated_norm_residual(float* res, const TY* y, const TG* gate,
 template <typename T>
 void launch_norm_sigmoid_gate(T* out, const float* o, const float* w,
                               const T* gate, float eps, int rows, int n,
-                              long gate_stride, hipStream_t st) {
+                              long gate_stride, int gate_cols,
+                              hipStream_t st) {
   if (rows == 0) return;
   hipLaunchKernelGGL((norm_sigmoid_gate_kernel<T>), dim3(rows), dim3(256), 0,
-                     st, out, o, w, gate, eps, n, gate_stride);
+                     st, out, o, w, gate, eps, n, gate_stride, gate_cols);
+}
+template <typename T>
+void launch_norm_residual_add(float* res, T* h, const T* y, const float* w1,
+                              float eps, int rows, int width, long y_stride,
+                              hipStream_t st) {
+  if (rows == 0) return;
+  hipLaunchKernelGGL((norm_residual_add_kernel<T>), dim3(rows), dim3(256), 0,
+                     st, res, h, y, w1, eps, width, y_stride);
 }
 template <typename T>
 void launch_gated_group_norm(T* out, const float* o, const float* w,
@@ -215,8 +260,17 @@ void launch_silu_mul(T* out, const T* x, long rows, int F, hipStream_t st) {
   const long n = rows * (long)F;
   if (n == 0) return;
   const int blocks = (int)((n + 255) / 256 < 65535 ? (n + 255) / 256 : 65535);
-  hipLaunchKernelGGL((silu_mul_kernel<T>), dim3(blocks), dim3(256), 0, st,
-                     out, x, rows, F);
+  hipLaunchKernelGGL((act_mul_kernel<T, false>), dim3(blocks), dim3(256), 0,
+                     st, out, x, rows, F);
+}
+template <typename T>
+void launch_gelu_tanh_mul(T* out, const T* x, long rows, int F,
+                          hipStream_t st) {
+  const long n = rows * (long)F;
+  if (n == 0) return;
+  const int blocks = (int)((n + 255) / 256 < 65535 ? (n + 255) / 256 : 65535);
+  hipLaunchKernelGGL((act_mul_kernel<T, true>), dim3(blocks), dim3(256), 0,
+                     st, out, x, rows, F);
 }
 template <typename T>
 void launch_rope_interleaved(T* x, const long* pos, const double* inv_freq,
@@ -234,8 +288,13 @@ void launch_rope_interleaved(T* x, const long* pos, const double* inv_freq,
 #define INST_NORMS(T)                                                         \
   template void launch_norm_sigmoid_gate<T>(T*, const float*, const float*,   \
                                             const T*, float, int, int, long,  \
-                                            hipStream_t);                     \
+                                            int, hipStream_t);                \
+  template void launch_norm_residual_add<T>(float*, T*, const T*,             \
+                                            const float*, float, int, int,    \
+                                            long, hipStream_t);               \
   template void launch_silu_mul<T>(T*, const T*, long, int, hipStream_t);     \
+  template void launch_gelu_tanh_mul<T>(T*, const T*, long, int,              \
+                                        hipStream_t);                         \
   template void launch_gated_group_norm<T>(T*, const float*, const float*,    \
                                            int, const T*, long, float, int,   \
                                            int, int, int, int, hipStream_t);  \
