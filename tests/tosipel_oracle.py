@@ -85,6 +85,39 @@ def o_conv(u, w):
     return out
 
 
+def o_attend(q, keys, values, scale, sink=None):
+    """One query vector against the keys it sees: softmax(scale q.k) v,
+    with exp(sink) as one more term of the denominator when given."""
+    s = (keys @ q) * scale
+    m = float(s.max()) if sink is None else max(float(s.max()), float(sink))
+    e = torch.exp(s - m)
+    den = e.sum() + (0.0 if sink is None else math.exp(float(sink) - m))
+    return (e / den) @ values
+
+
+def o_delta_core(q, k, v, b, a, A_log, dt_bias, S=None):
+    """q, k [T, G, D] and v [T, H, Dv] after convolution and silu, b and a
+    [T, H] as projected. Returns the read-outs [T, H, Dv] and the state
+    [H, D, Dv] after the last token."""
+    T, G, D = q.shape
+    H, Dv = v.shape[1], v.shape[2]
+    per = H // G
+    q = q / torch.sqrt((q ** 2).sum(-1, keepdim=True) + 1e-6) * D ** -0.5
+    k = k / torch.sqrt((k ** 2).sum(-1, keepdim=True) + 1e-6)
+    beta = o_sigmoid(b)
+    g = torch.exp(-torch.exp(A_log) * o_softplus(a + dt_bias))
+    S = torch.zeros(H, D, Dv, dtype=F64) if S is None else S.clone()
+    o = torch.zeros(T, H, Dv, dtype=F64)
+    for t in range(T):
+        for n in range(H):
+            kk, qq = k[t, n // per], q[t, n // per]
+            S[n] = g[t, n] * S[n]
+            u = beta[t, n] * (v[t, n] - S[n].T @ kk)
+            S[n] = S[n] + torch.outer(kk, u)
+            o[t, n] = S[n].T @ qq
+    return o, S
+
+
 def o_window_attention(Wt, p, mc, h, eps):
     T = h.shape[0]
     H, G, D, Dv = mc["heads"], mc["kv_heads"], mc["dim"], mc["vdim"]
@@ -107,11 +140,8 @@ def o_window_attention(Wt, p, mc, h, eps):
         lo = max(0, t - size + 1)
         for a in range(H):
             kv = a // per
-            s = (k[lo:t + 1, kv] @ q[t, a]) * mc["scale"]
-            m = max(float(s.max()), float(Wt[p + "sink"][a]))
-            e = torch.exp(s - m)
-            den = e.sum() + math.exp(float(Wt[p + "sink"][a]) - m)
-            out[t, a] = (e / den) @ v[lo:t + 1, kv] * gate[t, a]
+            out[t, a] = o_attend(q[t, a], k[lo:t + 1, kv], v[lo:t + 1, kv],
+                                 mc["scale"], Wt[p + "sink"][a]) * gate[t, a]
     return out.reshape(T, H * Dv) @ Wt[p + "o"].T
 
 
@@ -126,32 +156,19 @@ def o_latent_attention(Wt, p, mc, h, eps):
     out = torch.zeros(T, H, Dv, dtype=F64)
     for t in range(T):
         for a in range(H):
-            s = (k[:t + 1, a] @ q[t, a]) * mc["scale"]
-            out[t, a] = torch.softmax(s, 0) @ v[:t + 1, a]
+            out[t, a] = o_attend(q[t, a], k[:t + 1, a], v[:t + 1, a],
+                                 mc["scale"])
     return out.reshape(T, H * Dv) @ Wt[p + "o"].T
 
 
 def o_delta(Wt, p, mc, h, eps):
     T = h.shape[0]
     H, G, D, Dv = mc["heads"], mc["kv_heads"], mc["dim"], mc["vdim"]
-    per = H // G
     q = o_silu(o_conv(h @ Wt[p + "q"].T, Wt[p + "q.conv"])).view(T, G, D)
     k = o_silu(o_conv(h @ Wt[p + "k"].T, Wt[p + "k.conv"])).view(T, G, D)
     v = o_silu(o_conv(h @ Wt[p + "v"].T, Wt[p + "v.conv"])).view(T, H, Dv)
-    q = q / torch.sqrt((q ** 2).sum(-1, keepdim=True) + 1e-6) * D ** -0.5
-    k = k / torch.sqrt((k ** 2).sum(-1, keepdim=True) + 1e-6)
-    beta = o_sigmoid(h @ Wt[p + "b"].T)                      # [T, H]
-    g = torch.exp(-torch.exp(Wt[p + "A_log"])
-                  * o_softplus(h @ Wt[p + "a"].T + Wt[p + "dt_bias"]))
-    S = torch.zeros(H, D, Dv, dtype=F64)
-    o = torch.zeros(T, H, Dv, dtype=F64)
-    for t in range(T):
-        for a in range(H):
-            kk, qq = k[t, a // per], q[t, a // per]
-            S[a] = g[t, a] * S[a]
-            u = beta[t, a] * (v[t, a] - S[a].T @ kk)
-            S[a] = S[a] + torch.outer(kk, u)
-            o[t, a] = S[a].T @ qq
+    o, _ = o_delta_core(q, k, v, h @ Wt[p + "b"].T, h @ Wt[p + "a"].T,
+                        Wt[p + "A_log"], Wt[p + "dt_bias"])
     o = o_rms(o, eps) * Wt[p + "norm"]
     o = o.reshape(T, H * Dv) * o_silu(h @ Wt[p + "g"].T)
     return o @ Wt[p + "o"].T
@@ -174,7 +191,8 @@ def o_forward(cfg, Wt, tokens):
     x = Wt["embed"][torch.tensor(tokens)] * cfg["embedding"]["scale"]
     after = []
     for i, lc in enumerate(cfg["layers"]):
-        p = f"l{lc.get('weights_of', i)}."
+        j = lc.get("weights_of")
+        p = f"l{i if j is None else j}."
         x = x + o_rms(o_mixer(Wt, p, lc, x, eps), eps) * (1 + Wt[p + "norm1"])
         if lc.get("mlp") is not None:
             x = x + o_rms(o_ff(Wt, p + "mlp.", x), eps) * (1 + Wt[p + "norm2"])
