@@ -67,7 +67,7 @@ def parse_args():
                          "measurement, not the headline record)")
     ap.add_argument("--hybrid-sizes", default="2k,4k")
     ap.add_argument("--hybrid-family", default="pugovik",
-                    choices=("pugovik", "dunusun"),
+                    choices=("pugovik", "dunusun", "tosipel"),
                     help="which hybrid stack --mode hybrid measures beside "
                          "the equal-size llama stack")
     ap.add_argument("--model", default="llama-3-8b")
@@ -382,6 +382,189 @@ def _dunusun_kernels(size, device, T, batch, ctx):
     return out
 
 
+def _tosipel_kernels(size, device, T, batch, ctx):
+    """Achieved rates of the Tosipel mixer kernels at one layer's shapes,
+    beside the like kernels of the dunusun / pugovik / llama stacks of that
+    size."""
+    from xllm_service_amd import ops
+    from xllm_service_amd.models.config import get_config
+    from xllm_service_amd.ops import hybrid as hops
+    tc, dc, pc, lc = (get_config(f"{f}-{size}") for f in (
+        "tosipel", "dunusun", "pugovik", "llama"))
+    att = next(l.mixer for l in tc.layers if l.type == "attention")
+    lat = next(l.mixer for l in tc.layers if l.type == "latent_attention")
+    dl = next(l.mixer for l in tc.layers if l.type == "delta")
+    cap = next(l.mixer for l in dc.layers if l.type == "parallel")["left"]
+    ssm = next(l.mixer for l in dc.layers if l.type == "mamba2")
+    plat = next(l.mixer for l in pc.layers if l.type == "latent_attention")
+    bf = dict(dtype=torch.bfloat16, device=device)
+    f32 = dict(dtype=torch.float32, device=device)
+    i32 = dict(dtype=torch.int32, device=device)
+    out = []
+    nblk = (max(T, ctx) + 15) // 16
+    tab = torch.arange(batch * nblk, **i32).view(batch, nblk)
+    cu = torch.tensor([0, T], **i32)
+    sl = torch.tensor([T], **i32)
+    sld = torch.full((batch,), ctx, **i32)
+    z1 = torch.zeros(1, **i32)
+    sls = torch.arange(batch, **i32)
+    cx = torch.full((batch,), ctx, **i32)
+    # ---- windowed attention with a sink vs the soft-capped / llama kernels
+    H, G, D, Dv = att["heads"], att["kv_heads"], att["dim"], att["vdim"]
+    win = att["mask"]["size"]
+    kc = torch.randn(batch * nblk, G, 16, D, **bf)
+    vc = torch.randn(batch * nblk, G, 16, Dv, **bf)
+    q = torch.randn(T, H * D, **bf)
+    o = torch.empty(T, H, Dv, **f32)
+    sink = torch.zeros(H, **f32)
+    seen = sum(min(i + 1, win) for i in range(T))      # (query, key) pairs
+    t = _time_gpu(lambda: hops.capped_attn(q, kc, vc, tab[:1], cu, sl, H,
+                                           att["scale"], 0.0, o, window=win,
+                                           sink=sink), 3, 1)
+    out.append((f"window_attn prefill (window {win})", t,
+                2.0 * H * (D + Dv) * seen / t / 1e12, "TFLOP/s"))
+    qd = torch.randn(batch, H * D, **bf)
+    od = torch.empty(batch, H, Dv, **f32)
+    t = _time_gpu(lambda: hops.capped_attn(qd, kc, vc, tab, None, sld, H,
+                                           att["scale"], 0.0, od, window=win,
+                                           sink=sink))
+    out.append((f"window_attn decode (window {win})", t,
+                batch * min(ctx, win) * G * (D + Dv) * 2 / t / 1e9, "GB/s"))
+    Hc, Gc, Dc, Dvc = cap["heads"], cap["kv_heads"], cap["dim"], cap["vdim"]
+    kcc = torch.randn(batch * nblk, Gc, 16, Dc, **bf)
+    vcc = torch.randn(batch * nblk, Gc, 16, Dvc, **bf)
+    qc = torch.randn(T, Hc * Dc, **bf)
+    oc = torch.empty(T, Hc, Dvc, **f32)
+    t = _time_gpu(lambda: hops.capped_attn(qc, kcc, vcc, tab[:1], cu, sl, Hc,
+                                           cap["scale"], cap["softcap"], oc),
+                  3, 1)
+    out.append(("capped_attn prefill (dunusun)", t,
+                2.0 * Hc * (Dc + Dvc) * T * (T + 1) / 2 / t / 1e12,
+                "TFLOP/s"))
+    qcd = torch.randn(batch, Hc * Dc, **bf)
+    ocd = torch.empty(batch, Hc, Dvc, **f32)
+    t = _time_gpu(lambda: hops.capped_attn(qcd, kcc, vcc, tab, None, sld, Hc,
+                                           cap["scale"], cap["softcap"], ocd))
+    out.append(("capped_attn decode (dunusun)", t,
+                batch * ctx * Gc * (Dc + Dvc) * 2 / t / 1e9, "GB/s"))
+    Hq, Hk, Dl = lc.num_heads, lc.num_kv_heads, lc.head_dim
+    kl = torch.randn(batch * nblk, Hk, 16, Dl, **bf)
+    vl = torch.randn(batch * nblk, Hk, 16, Dl, **bf)
+    qld = torch.randn(batch, Hq, Dl, **bf)
+    t = _time_gpu(lambda: ops.paged_attn_decode(qld, kl, vl, tab, sld, 0.1))
+    out.append(("paged_attn decode (llama)", t,
+                batch * ctx * Hk * Dl * 2 * 2 / t / 1e9, "GB/s"))
+    # ---- latent attention without a rotated part vs pugovik's -------------
+    for label, Hh, r, rd in (
+            ("latent_attn", lat["heads"], lat["kv_rank"], 0),
+            ("latent_attn (pugovik)", plat["heads"], plat["kv_rank"],
+             plat["rot_dim"])):
+        Wl = r + rd
+        cache = torch.randn(batch * nblk, 16, Wl, **bf)
+        ql_ = torch.randn(T, Hh, Wl, **bf)
+        ol = torch.empty(T, Hh, r, **f32)
+        t = _time_gpu(lambda: hops.latent_attn(ql_, cache, tab[:1], cu, sl,
+                                               0.1, r, ol), 3, 1)
+        out.append((f"{label} prefill", t,
+                    2.0 * Hh * (Wl + r) * T * (T + 1) / 2 / t / 1e12,
+                    "TFLOP/s"))
+        qld_ = torch.randn(batch, Hh, Wl, **bf)
+        old = torch.empty(batch, Hh, r, **f32)
+        t = _time_gpu(lambda: hops.latent_attn(qld_, cache, tab, None, sld,
+                                               0.1, r, old))
+        out.append((f"{label} decode", t, batch * ctx * Wl * 2 / t / 1e9,
+                    "GB/s"))
+    # ---- delta rule vs the selective state space recurrence ---------------
+    Hh, Gg, Dk, Dvv = dl["heads"], dl["kv_heads"], dl["dim"], dl["vdim"]
+
+    def delta(tokens, slots, cuq, ctxl):
+        qq = torch.randn(tokens, Gg * Dk, **bf)
+        kk = torch.randn(tokens, Gg * Dk, **bf)
+        vv = torch.randn(tokens, Hh * Dvv, **bf)
+        bb, aa = torch.randn(tokens, Hh, **bf), torch.randn(tokens, Hh, **bf)
+        st = torch.zeros(batch, Hh, Dk, Dvv, **f32)
+        p = torch.zeros(Hh, **f32)
+        oo = torch.empty(tokens, Hh, Dvv, **f32)
+        return lambda: hops.delta_rule(qq, kk, vv, bb, aa, p, p, st, slots,
+                                       cuq, ctxl, Gg, oo, max_q_len=tokens)
+    t = _time_gpu(delta(T, z1, cu, z1), 3, 1)
+    out.append(("delta_rule prefill", t, 8.0 * Hh * Dk * Dvv * T / t / 1e12,
+                "TFLOP/s (recurrence form)"))
+    t = _time_gpu(delta(batch, sls, None, cx))
+    out.append(("delta_rule decode", t,
+                batch * Hh * Dk * Dvv * 4 * 2 / t / 1e9, "GB/s"))
+    Hs, P, N, Gs = ssm["heads"], ssm["vdim"], ssm["state"], ssm["groups"]
+
+    def recur(tokens, slots, cuq, ctxl):
+        qq = torch.randn(tokens, Gs * N, **bf)
+        kk = torch.randn(tokens, Gs * N, **bf)
+        vv = torch.randn(tokens, Hs * P, **bf)
+        gg = torch.randn(tokens, Hs, **bf)
+        st = torch.zeros(batch, Hs, N, P, **f32)
+        p0 = torch.zeros(Hs, **f32)
+        oo = torch.empty(tokens, Hs, P, **f32)
+        return lambda: hops.gated_recurrence(
+            0, qq, kk, vv, gg, p0, p0, p0, 0.06, 0.1, st, slots, cuq, ctxl,
+            Gs, oo, max_q_len=tokens)
+    t = _time_gpu(recur(T, z1, cu, z1), 3, 1)
+    out.append(("gated_recurrence ssm prefill (dunusun)", t,
+                4.0 * Hs * N * P * T / t / 1e12, "TFLOP/s (recurrence form)"))
+    t = _time_gpu(recur(batch, sls, None, cx))
+    out.append(("gated_recurrence ssm decode (dunusun)", t,
+                batch * Hs * N * P * 4 * 2 / t / 1e9, "GB/s"))
+    # ---- q/k preparation, convolution, norms, gates ------------------------
+    big = torch.randn(T, H * D + G * D + G * Dv, **bf)
+    qw, kw = torch.ones(H * D, **f32), torch.ones(G * D, **f32)
+    rot = att["rot"]["dims"]
+    inv = torch.ones(rot // 2, dtype=torch.float64, device=device)
+    pos = torch.arange(T, device=device)
+    slot = torch.arange(T, device=device)
+    t = _time_gpu(lambda: hops.rownorm_rope_store(
+        big[:, :H * D], big[:, H * D:H * D + G * D], big[:, H * D + G * D:],
+        qw, kw, 1e-6, pos, inv, rot, H, G, kc, vc, slot))
+    out.append(("rownorm_rope_store", t,
+                T * (H * D * 2 + G * D * 2 + G * Dv * 2) * 2 / t / 1e9,
+                "GB/s"))
+    C, taps = 2 * Gg * Dk + Hh * Dvv, dl["conv"]
+    xin = torch.randn(T, C, **bf)
+    cw = torch.randn(C, taps, **bf)
+    cst = torch.zeros(batch, taps - 1, C, **bf)
+    t = _time_gpu(lambda: hops.short_conv(xin, cw, None, cst, 0, z1, cu, z1,
+                                          1, C, act_silu=True))
+    out.append(("short_conv+silu", t, T * C * 4 / t / 1e9, "GB/s"))
+    Wd = tc.hidden_size
+    x1 = torch.randn(T, Wd, **f32)
+    y = torch.randn(T, Wd, **bf)
+    w = torch.ones(Wd, **f32)
+    t = _time_gpu(lambda: hops.norm_residual_add_(x1, y, w, 1e-6,
+                                                  torch.bfloat16))
+    out.append(("norm_residual_add", t, T * Wd * 12 / t / 1e9, "GB/s"))
+    xd1, yd1 = x1[:batch].contiguous(), y[:batch].contiguous()
+    t = _time_gpu(lambda: hops.norm_residual_add_(xd1, yd1, w, 1e-6,
+                                                  torch.bfloat16))
+    out.append((f"norm_residual_add, {batch} rows (decode)", t,
+                batch * Wd * 12 / t / 1e9, "GB/s"))
+    S = dc.streams or 1
+    xs = torch.randn(T, S, Wd, **f32)
+    wi, mix = torch.ones(S, **f32), torch.eye(S, **f32)
+    t = _time_gpu(lambda: hops.streams_update_mix_norm_(
+        xs, mix, wi, y, 1.0, y, 1.0, wi, w, w, 1e-6))
+    out.append(("streams_update_mix_norm (dunusun)", t,
+                T * Wd * (8 * S + 6) / t / 1e9, "GB/s"))
+    gt = torch.randn(T, Wd, **bf)
+    t = _time_gpu(lambda: hops.gated_norm_residual(x1, y, gt, w, w, w, 0.5,
+                                                   1e-6, pc.norm_groups))
+    out.append(("gated_norm_residual (pugovik)", t, T * Wd * 12 / t / 1e9,
+                "GB/s"))
+    ff = next(l.mlp for l in tc.layers if l.mlp)["ff"]
+    gu = torch.randn(T, 2 * ff, **bf)
+    t = _time_gpu(lambda: hops.gelu_tanh_mul(gu))
+    out.append(("gelu_tanh_mul", t, T * ff * 6 / t / 1e9, "GB/s"))
+    t = _time_gpu(lambda: hops.silu_mul(gu))
+    out.append(("silu_mul (pugovik)", t, T * ff * 6 / t / 1e9, "GB/s"))
+    return out
+
+
 def run_hybrid_mode(args, device):
     assert torch.cuda.is_available(), "hybrid mode measures the HIP path"
     kernels = _hybrid_kernels
@@ -389,6 +572,9 @@ def run_hybrid_mode(args, device):
     if args.hybrid_family == "dunusun":
         kernels = _dunusun_kernels
         fams = ("dunusun", "pugovik", "llama")
+    if args.hybrid_family == "tosipel":
+        kernels = _tosipel_kernels
+        fams = ("tosipel", "dunusun", "llama")
     for size in args.hybrid_sizes.split(","):
         T, batch, ctx = 4096, 32, 2048
         for name, t, rate, unit in kernels(size, device, T, batch, ctx):

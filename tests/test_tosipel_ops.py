@@ -344,6 +344,43 @@ def test_delta_rule_through_portions_and_slots(target, H, G, D, Dv):
 
 
 @pytest.mark.parametrize("target", TARGETS)
+@pytest.mark.parametrize("H,G,D,Dv", [(2, 1, 40, 12), (4, 2, 64, 64),
+                                      (2, 2, 128, 128), (3, 1, 16, 100)])
+def test_delta_rule_long_chunks(target, H, G, D, Dv):
+    """Chunks long enough for the piece-parallel passes (pieces of 128
+    tokens, the last one short), from a zero state and from a carried one,
+    beside a short request in the same call."""
+    dev, dt = target
+    g = torch.Generator().manual_seed(D + Dv)
+    T = 650
+    q, k, v, b, a = _delta_inputs(g, T, H, G, D, Dv, dt)
+    A_log = torch.randn(H, generator=g) * 0.5 - 2.0
+    dt_bias = torch.randn(H, generator=g)
+    want, S_end = o_delta_core(
+        q.to(F64).view(T, G, D), k.to(F64).view(T, G, D),
+        v.to(F64).view(T, H, Dv), b.to(F64), a.to(F64), A_log.to(F64),
+        dt_bias.to(F64))
+    dq, dk, dv, db, da = (x.to(dev) for x in (q, k, v, b, a))
+    for cuts in ([T], [37, T - 37]):
+        state = torch.randn(3, H, D, Dv, generator=g).to(dev)   # stale
+        out = torch.empty(T, H, Dv, device=dev)
+        at = 0
+        for n in cuts:
+            # the short request (rows 0..4 again, no slot) comes first
+            sel = list(range(5)) + list(range(at, at + n))
+            o = torch.empty(n + 5, H, Dv, device=dev)
+            hops.delta_rule(dq[sel], dk[sel], dv[sel], db[sel], da[sel],
+                            dt_bias.to(dev), A_log.to(dev), state,
+                            _i32([-1, 2], dev), _i32([0, 5, n + 5], dev),
+                            _i32([0, at], dev), G, o, max_q_len=n)
+            out[at:at + n] = o[5:]
+            _close(o[:5], want[:5], target, ("short", cuts), 5)
+            at += n
+        _close(out, want, target, cuts, 10)
+        _close(state[2], S_end, target, ("state", cuts), 10)
+
+
+@pytest.mark.parametrize("target", TARGETS)
 def test_delta_rule_long_decoding_batch(target):
     """Four sequences decode 120 tokens each, one row per sequence and call
     (the whole-state kernel), after prompts of unequal length."""

@@ -39,7 +39,8 @@ template <typename T>
 void launch_delta_rule(float*, const T*, const T*, const T*, const T*,
                        const T*, long, long, long, long, long, const float*,
                        const float*, float*, const int*, const int*,
-                       const int*, int, int, int, int, int, hipStream_t);
+                       const int*, int, int, int, int, int, int, int, float*,
+                       hipStream_t);
 template <typename T>
 void launch_rope_interleaved(T*, const long*, const double*, float, int, int,
                              int, long, long, int, hipStream_t);
@@ -272,7 +273,8 @@ void rownorm_rope_store(Tensor q_out, Tensor q, Tensor k, Tensor v, Tensor wq,
 // v [T, H*Dv], b/a [T, H] row views (after convolution: q, k, v)
 void delta_rule(Tensor out, Tensor q, Tensor k, Tensor v, Tensor b, Tensor a,
                 Tensor dt_bias, Tensor A_log, Tensor state, Tensor slots,
-                c10::optional<Tensor> cu_q, Tensor ctx_lens, long groups) {
+                c10::optional<Tensor> cu_q, Tensor ctx_lens, long groups,
+                long max_q_len) {
   CHK_F32C(out); CHK_ACT(q); CHK_ACT(k); CHK_ACT(v); CHK_ACT(b); CHK_ACT(a);
   CHK_F32C(dt_bias); CHK_F32C(A_log); CHK_F32C(state); CHK_I32C(slots);
   CHK_I32C(ctx_lens);
@@ -300,10 +302,30 @@ void delta_rule(Tensor out, Tensor q, Tensor k, Tensor v, Tensor b, Tensor a,
   } else {
     TORCH_CHECK(n_seqs == T, "decode: one sequence per token");
   }
+  // long chunks on a chip that the (sequence, head) pairs alone leave mostly
+  // empty: piece-parallel passes (three times the arithmetic, many times the
+  // workgroups). XLLM_DELTA_CHUNK: piece length, 0 switches the passes off.
+  int chunk = 128, max_chunks = 1;
+  Tensor ws;
+  if (cu != nullptr) {
+    const long bound = max_q_len > 0 ? std::min<long>(max_q_len, T) : T;
+    if (const char* e = std::getenv("XLLM_DELTA_CHUNK"))
+      chunk = std::min(1024, std::max(0, std::atoi(e)));
+    const long rec = (long)H * D * (Dv + D) * 4;
+    while (chunk > 0 && (bound + chunk - 1) / chunk * n_seqs * rec > (1L << 31))
+      chunk *= 2;                             // keep the scratch under 2 GiB
+    const long wgs = (long)n_seqs * H * ((Dv + 63) / 64);
+    if (chunk > 0 && bound >= 4L * chunk && wgs < 512) {
+      max_chunks = (int)((bound + chunk - 1) / chunk);
+      ws = torch::empty({(long)n_seqs * max_chunks, (long)H, (long)D,
+                         (long)(Dv + D)}, state.options());
+    }
+  }
+  float* wsp = max_chunks > 1 ? ptr<float>(ws) : nullptr;
   if (is_f32(q))
-    hy::launch_delta_rule<float>(ptr<float>(out), ptr<float>(q), ptr<float>(k), ptr<float>(v), ptr<float>(b), ptr<float>(a), q.stride(0), k.stride(0), v.stride(0), b.stride(0), a.stride(0), ptr<float>(dt_bias), ptr<float>(A_log), ptr<float>(state), ptr<int>(slots), cu, ptr<int>(ctx_lens), n_seqs, H, groups, D, Dv, cur());
+    hy::launch_delta_rule<float>(ptr<float>(out), ptr<float>(q), ptr<float>(k), ptr<float>(v), ptr<float>(b), ptr<float>(a), q.stride(0), k.stride(0), v.stride(0), b.stride(0), a.stride(0), ptr<float>(dt_bias), ptr<float>(A_log), ptr<float>(state), ptr<int>(slots), cu, ptr<int>(ctx_lens), n_seqs, H, groups, D, Dv, chunk, max_chunks, wsp, cur());
   else
-    hy::launch_delta_rule<bf>(ptr<float>(out), ptr<bf>(q), ptr<bf>(k), ptr<bf>(v), ptr<bf>(b), ptr<bf>(a), q.stride(0), k.stride(0), v.stride(0), b.stride(0), a.stride(0), ptr<float>(dt_bias), ptr<float>(A_log), ptr<float>(state), ptr<int>(slots), cu, ptr<int>(ctx_lens), n_seqs, H, groups, D, Dv, cur());
+    hy::launch_delta_rule<bf>(ptr<float>(out), ptr<bf>(q), ptr<bf>(k), ptr<bf>(v), ptr<bf>(b), ptr<bf>(a), q.stride(0), k.stride(0), v.stride(0), b.stride(0), a.stride(0), ptr<float>(dt_bias), ptr<float>(A_log), ptr<float>(state), ptr<int>(slots), cu, ptr<int>(ctx_lens), n_seqs, H, groups, D, Dv, chunk, max_chunks, wsp, cur());
 }
 
 void silu_mul(Tensor out, Tensor x) {

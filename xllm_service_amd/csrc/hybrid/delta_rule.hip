@@ -23,6 +23,19 @@
 // lanes of a column group sum their partial a and c by DPP. Decode: one
 // workgroup per (sequence, head) holds the whole state in registers as
 // float4 row pieces and sums the row groups' partials through LDS.
+//
+// Long chunks run piece-parallel. A token maps the state linearly,
+//   S <- g (I - beta k k^T) S + beta k v^T,
+// so a piece of tokens maps S to M S + N with M [D, D] the product of its
+// token matrices and N [D, Dv] what the piece builds from a zero state. M is
+// what the same recurrence makes of an identity state with zero values:
+// pass 1 runs every piece over Dv + D columns ([zero | identity] in,
+// [N | M] out), a scan applies S <- M S + N piece after piece on the fp32
+// matrix pipe (v_mfma_f32_16x16x4_f32, true 32-bit products) and leaves the
+// state BEFORE each piece in N's place, pass 2 reruns the pieces from these
+// states and writes the outputs.
+#include <cstdlib>
+
 #include "hybrid_common.h"
 
 namespace xllm {
@@ -68,11 +81,18 @@ XLLM_DEV void dr_gates(const DRArgs<T>& A, long row, int h, float* g,
   *beta = 1.0f / (1.0f + expf(-IO<T>::ld(A.b + row * A.b_stride + h)));
 }
 
+// mode 0: the whole chunk of a sequence in one workgroup (slot in and out)
+// mode 1: tokens [c*chunk, (c+1)*chunk) over Dv + D columns from [0 | I], no
+//         outputs; [N | M] goes to the piece's record in ws
+//         ([s*max_chunks + c][h][D][Dv + D])
+// mode 2: the same tokens from the state the scan left in the record's first
+//         Dv columns; outputs written, nothing stored
 template <typename T, int CPT>
 __global__ void __launch_bounds__(256) delta_rule_kernel(
     float* __restrict__ out, DRArgs<T> A, float* __restrict__ state,
     const int* __restrict__ slots, const int* __restrict__ cu_q,
-    const int* __restrict__ ctx_lens) {
+    const int* __restrict__ ctx_lens, int mode, int chunk, int max_chunks,
+    float* __restrict__ ws) {
   extern __shared__ float smem[];
   constexpr int VS = DR_CG * CPT;         // value columns per workgroup
   const int D = A.D, Dv = A.Dv, heads = A.heads;
@@ -81,13 +101,22 @@ __global__ void __launch_bounds__(256) delta_rule_kernel(
   float* vs = ks + DR_TC * D;             // [TC][VS]
   float* sc = vs + DR_TC * VS;            // [TC][NS]
 
-  const int s = blockIdx.x, h = blockIdx.y, v0 = blockIdx.z * VS;
+  const int s = blockIdx.x / max_chunks, cidx = blockIdx.x % max_chunks;
+  const int h = blockIdx.y, v0 = blockIdx.z * VS;
   const int kg = h / (heads / A.groups);
   const int tid = threadIdx.x;
   const int j = tid / DR_R, r = tid % DR_R;
   const int col = v0 + j * CPT;           // first of this thread's columns
-  const int t0 = cu_q ? cu_q[s] : s;
-  const int t1 = cu_q ? cu_q[s + 1] : s + 1;
+  int t0 = cu_q ? cu_q[s] : s;
+  int t1 = cu_q ? cu_q[s + 1] : s + 1;
+  if (mode != 0) {
+    t0 += cidx * chunk;
+    if (t0 >= t1) return;                 // uniform for the workgroup
+    t1 = min(t1, t0 + chunk);
+  }
+  const int E = Dv + D;                   // columns of a piece record
+  const int ncols = mode == 1 ? E : Dv;   // columns this launch covers
+  const int rs = mode == 0 ? Dv : E;      // row stride of what sp points at
   const int slot = slots[s];
   const int M = (D + DR_R - 1) / DR_R;
   const float qmul = 1.0f / sqrtf((float)D);
@@ -99,8 +128,13 @@ __global__ void __launch_bounds__(256) delta_rule_kernel(
     for (int c = 0; c < CPT; ++c) S[m][c] = 0.f;
   float* sp = (slot >= 0)
       ? state + (((long)slot * heads + h) * D) * (long)Dv : nullptr;
-  const bool load = sp && ctx_lens[s] > 0;
-  const bool vec = CPT == 4 && (Dv & 3) == 0 && col + 3 < Dv;
+  bool load = sp && ctx_lens[s] > 0;
+  if (mode != 0) {
+    sp = ws + ((((long)s * max_chunks + cidx) * heads + h) * D) * (long)E;
+    load = mode == 2;
+  }
+  const bool vec = CPT == 4 && (Dv & 3) == 0 && (rs & 3) == 0 &&
+                   col + 3 < ncols;
   if (load) {
 #pragma unroll
     for (int m = 0; m < DR_MAXM; ++m) {
@@ -108,16 +142,23 @@ __global__ void __launch_bounds__(256) delta_rule_kernel(
       if (m < M && i < D) {
         if (vec) {
           const float4 x = *reinterpret_cast<const float4*>(
-              sp + (long)i * Dv + col);
+              sp + (long)i * rs + col);
           S[m][0] = x.x; S[m][CPT > 1 ? 1 : 0] = x.y;
           S[m][CPT > 2 ? 2 : 0] = x.z; S[m][CPT > 3 ? 3 : 0] = x.w;
         } else {
 #pragma unroll
           for (int c = 0; c < CPT; ++c)
-            if (col + c < Dv) S[m][c] = sp[(long)i * Dv + col + c];
+            if (col + c < ncols) S[m][c] = sp[(long)i * rs + col + c];
         }
       }
     }
+  }
+  if (mode == 1) {                        // identity under the M columns
+#pragma unroll
+    for (int m = 0; m < DR_MAXM; ++m)
+#pragma unroll
+      for (int c = 0; c < CPT; ++c)
+        if (col + c - Dv == r + DR_R * m) S[m][c] = 1.f;
   }
 
   for (int tb = t0; tb < t1; tb += DR_TC) {
@@ -193,7 +234,7 @@ __global__ void __launch_bounds__(256) delta_rule_kernel(
           for (int c = 0; c < CPT; ++c) S[m][c] = g * S[m][c] + kk * uk[c];
         }
       }
-      if (r == 0) {
+      if (mode != 1 && r == 0) {
         float* op = out + ((long)(tb + tt) * heads + h) * Dv + col;
 #pragma unroll
         for (int c = 0; c < CPT; ++c)
@@ -201,23 +242,119 @@ __global__ void __launch_bounds__(256) delta_rule_kernel(
       }
     }
   }
-  if (sp) {
+  if (sp && mode != 2) {
 #pragma unroll
     for (int m = 0; m < DR_MAXM; ++m) {
       const int i = r + DR_R * m;
       if (m < M && i < D) {
         if (vec) {
-          *reinterpret_cast<float4*>(sp + (long)i * Dv + col) = make_float4(
+          *reinterpret_cast<float4*>(sp + (long)i * rs + col) = make_float4(
               S[m][0], S[m][CPT > 1 ? 1 : 0], S[m][CPT > 2 ? 2 : 0],
               S[m][CPT > 3 ? 3 : 0]);
         } else {
 #pragma unroll
           for (int c = 0; c < CPT; ++c)
-            if (col + c < Dv) sp[(long)i * Dv + col + c] = S[m][c];
+            if (col + c < ncols) sp[(long)i * rs + col + c] = S[m][c];
         }
       }
     }
   }
+}
+
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float dr_f32x4;
+
+// S <- M_c S + N_c over the pieces of a sequence, for 16 columns of one head.
+// S sits in LDS as [rows][16]; a wave owns every fourth 16-row tile of the
+// result. v_mfma_f32_16x16x4_f32: lane l gives A[l & 15][l >> 4] and
+// B[l >> 4][l & 15] and holds C[(l >> 4) * 4 + r][l & 15]. Within a block of
+// 16 inner indices lane group g takes the indices 4g..4g+3 (one 16 B load of
+// its M row), the same permutation on both operands. The record's first Dv
+// columns (N) are overwritten with the state before the piece.
+__global__ void __launch_bounds__(256) delta_rule_scan_kernel(
+    float* __restrict__ ws, float* __restrict__ state,
+    const int* __restrict__ slots, const int* __restrict__ cu_q,
+    const int* __restrict__ ctx_lens, int heads, int D, int Dv, int chunk,
+    int max_chunks) {
+  extern __shared__ float Sl[];           // [Dp][16]
+  const int s = blockIdx.x, h = blockIdx.y, col0 = blockIdx.z * 16;
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int n = lane & 15, g = lane >> 4;
+  const int E = Dv + D;
+  const int qlen = cu_q[s + 1] - cu_q[s];
+  const int n_chunks = (qlen + chunk - 1) / chunk;
+  const int slot = slots[s];
+  const int n_tiles = (D + 15) >> 4, Dp = n_tiles << 4;
+  const bool col_ok = col0 + n < Dv;
+  const bool from_slot = slot >= 0 && ctx_lens[s] > 0;
+  float* sst = state + (((long)max(slot, 0) * heads + h) * D) * (long)Dv;
+  for (int idx = tid; idx < Dp * 16; idx += 256) {
+    const int i = idx >> 4, jj = idx & 15;
+    Sl[idx] = (from_slot && i < D && col0 + jj < Dv)
+        ? sst[(long)i * Dv + col0 + jj] : 0.f;
+  }
+  __syncthreads();
+  const bool fast = (D & 15) == 0 && (E & 3) == 0 && (Dv & 3) == 0;
+  constexpr int MAXT = 4;                 // D <= 256: 16 tiles over 4 waves
+  for (int c = 0; c < n_chunks; ++c) {
+    float* rec = ws + ((((long)s * max_chunks + c) * heads + h) * D) * (long)E;
+    dr_f32x4 acc[MAXT];
+#pragma unroll
+    for (int tt = 0; tt < MAXT; ++tt) {
+      const int it = wv + 4 * tt;
+      acc[tt] = dr_f32x4{0.f, 0.f, 0.f, 0.f};
+      if (it >= n_tiles) continue;        // uniform per wave
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr) {
+        const int i = it * 16 + 4 * g + rr;
+        if (i < D && col_ok) acc[tt][rr] = rec[(long)i * E + col0 + n];
+      }
+      const int ia = it * 16 + n;
+      const float* mrow = rec + (long)min(ia, D - 1) * E + Dv;
+      for (int kb = 0; kb < D; kb += 16) {
+        float a4[4];
+        if (fast) {
+          const float4 x = *reinterpret_cast<const float4*>(mrow + kb + 4 * g);
+          a4[0] = x.x; a4[1] = x.y; a4[2] = x.z; a4[3] = x.w;
+        } else {
+#pragma unroll
+          for (int q4 = 0; q4 < 4; ++q4) {
+            const int ka = kb + 4 * g + q4;
+            a4[q4] = (ia < D && ka < D) ? mrow[ka] : 0.f;
+          }
+        }
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+          const int kk = kb + 4 * g + q4;            // < Dp
+          acc[tt] = __builtin_amdgcn_mfma_f32_16x16x4f32(
+              a4[q4], Sl[kk * 16 + n], acc[tt], 0, 0, 0);
+        }
+      }
+      // the state before this piece takes N's place (same thread, same
+      // elements it has just read)
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr) {
+        const int i = it * 16 + 4 * g + rr;
+        if (i < D && col_ok) rec[(long)i * E + col0 + n] = Sl[i * 16 + n];
+      }
+    }
+    __syncthreads();                      // every wave is done reading Sl
+#pragma unroll
+    for (int tt = 0; tt < MAXT; ++tt) {
+      const int it = wv + 4 * tt;
+      if (it >= n_tiles) continue;
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr) {
+        const int i = it * 16 + 4 * g + rr;
+        Sl[i * 16 + n] = (i < D && col_ok) ? acc[tt][rr] : 0.f;
+      }
+    }
+    __syncthreads();
+  }
+  if (slot >= 0)
+    for (int idx = tid; idx < Dp * 16; idx += 256) {
+      const int i = idx >> 4, jj = idx & 15;
+      if (i < D && col0 + jj < Dv) sst[(long)i * Dv + col0 + jj] = Sl[idx];
+    }
 }
 
 // Decode (one token per sequence): thread (rg, tc) owns columns 4tc..4tc+3 of
@@ -320,13 +457,33 @@ __global__ void __launch_bounds__(256) delta_rule_decode_kernel(
 template <typename T, int CPT>
 void launch_delta_rule_cpt(float* out, const DRArgs<T>& A, float* state,
                            const int* slots, const int* cu_q,
-                           const int* ctx_lens, int n_seqs, hipStream_t st) {
+                           const int* ctx_lens, int n_seqs, int chunk,
+                           int max_chunks, float* ws, hipStream_t st) {
   constexpr int VS = DR_CG * CPT;
-  const size_t lds = (size_t)(2 * DR_TC * A.D + DR_TC * VS + DR_TC * DR_NS) *
+  const int D = A.D, Dv = A.Dv;
+  const size_t lds = (size_t)(2 * DR_TC * D + DR_TC * VS + DR_TC * DR_NS) *
                      sizeof(float);
-  const int vz = (A.Dv + VS - 1) / VS;
-  hipLaunchKernelGGL((delta_rule_kernel<T, CPT>), dim3(n_seqs, A.heads, vz),
-                     dim3(256), lds, st, out, A, state, slots, cu_q, ctx_lens);
+  const int vz = (Dv + VS - 1) / VS;
+  if (ws == nullptr || max_chunks <= 1) {
+    hipLaunchKernelGGL((delta_rule_kernel<T, CPT>), dim3(n_seqs, A.heads, vz),
+                       dim3(256), lds, st, out, A, state, slots, cu_q,
+                       ctx_lens, 0, 0, 1, nullptr);
+    return;
+  }
+  const int vz1 = (Dv + D + VS - 1) / VS;
+  hipLaunchKernelGGL((delta_rule_kernel<T, CPT>),
+                     dim3(n_seqs * max_chunks, A.heads, vz1), dim3(256), lds,
+                     st, out, A, state, slots, cu_q, ctx_lens, 1, chunk,
+                     max_chunks, ws);
+  const int Dp = ((D + 15) >> 4) << 4;
+  hipLaunchKernelGGL(delta_rule_scan_kernel,
+                     dim3(n_seqs, A.heads, (Dv + 15) / 16), dim3(256),
+                     (size_t)Dp * 16 * sizeof(float), st, ws, state, slots,
+                     cu_q, ctx_lens, A.heads, D, Dv, chunk, max_chunks);
+  hipLaunchKernelGGL((delta_rule_kernel<T, CPT>),
+                     dim3(n_seqs * max_chunks, A.heads, vz), dim3(256), lds,
+                     st, out, A, state, slots, cu_q, ctx_lens, 2, chunk,
+                     max_chunks, ws);
 }
 
 template <typename T>
@@ -336,7 +493,7 @@ void launch_delta_rule(float* out, const T* q, const T* k, const T* v,
                        const float* dt_bias, const float* A_log, float* state,
                        const int* slots, const int* cu_q, const int* ctx_lens,
                        int n_seqs, int heads, int groups, int D, int Dv,
-                       hipStream_t st) {
+                       int chunk, int max_chunks, float* ws, hipStream_t st) {
   if (n_seqs == 0) return;
   DRArgs<T> A{q, k, v, b, a, q_stride, k_stride, v_stride, b_stride, a_stride,
               dt_bias, A_log, heads, groups, D, Dv};
@@ -357,21 +514,25 @@ void launch_delta_rule(float* out, const T* q, const T* k, const T* v,
       return;
     }
   }
-  // wide values and enough workgroups: four columns per thread
-  const bool wide = Dv >= 48 && (long)n_seqs * heads * ((Dv + 63) / 64) >= 256;
+  // wide values and enough workgroups: four columns per thread.
+  // XLLM_DELTA_COLS=1|4 fixes the choice (tuning knob).
+  bool wide = Dv >= 48 &&
+      (long)n_seqs * max_chunks * heads * ((Dv + 63) / 64) >= 256;
+  if (const char* e = std::getenv("XLLM_DELTA_COLS")) wide = e[0] == '4';
   if (wide)
     launch_delta_rule_cpt<T, 4>(out, A, state, slots, cu_q, ctx_lens, n_seqs,
-                                st);
+                                chunk, max_chunks, ws, st);
   else
     launch_delta_rule_cpt<T, 1>(out, A, state, slots, cu_q, ctx_lens, n_seqs,
-                                st);
+                                chunk, max_chunks, ws, st);
 }
 
 #define INST_DR(T)                                                            \
   template void launch_delta_rule<T>(                                         \
       float*, const T*, const T*, const T*, const T*, const T*, long, long,   \
       long, long, long, const float*, const float*, float*, const int*,       \
-      const int*, const int*, int, int, int, int, int, hipStream_t);
+      const int*, const int*, int, int, int, int, int, int, int, float*,      \
+      hipStream_t);
 INST_DR(float)
 INST_DR(unsigned short)
 

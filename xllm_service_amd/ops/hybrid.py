@@ -312,10 +312,11 @@ def rownorm_rope_store(q, k, v, q_w, k_w, eps: float, positions, inv_freq,
 def delta_rule(q, k, v, b, a, dt_bias, A_log, state, slots, cu_q, ctx_lens,
                groups: int, out, max_q_len: int = 0):
     """out fp32 [T, H, Dv] (written); see ref.delta_rule. q/k/v/b/a are row
-    views of the projections; state fp32 [slots, H, D, Dv] in place."""
+    views of the projections; state fp32 [slots, H, D, Dv] in place.
+    max_q_len: host-known bound on the longest sequence chunk (0: unknown)."""
     if q.is_cuda:
         _hyb().delta_rule(out, q, k, v, b, a, dt_bias, A_log, state, slots,
-                          cu_q, ctx_lens, groups)
+                          cu_q, ctx_lens, groups, max_q_len)
         return out
     out.copy_(ref.delta_rule(q, k, v, b, a, dt_bias, A_log, state, slots,
                              cu_q, ctx_lens, groups))
