@@ -312,6 +312,10 @@ void delta_rule(Tensor out, Tensor q, Tensor k, Tensor v, Tensor b, Tensor a,
     if (const char* e = std::getenv("XLLM_DELTA_CHUNK"))
       chunk = std::min(1024, std::max(0, std::atoi(e)));
     const long rec = (long)H * D * (Dv + D) * 4;
+    // shorter pieces while the first pass would not fill the chip
+    while (chunk > 32 && (bound + chunk - 1) / chunk * n_seqs * H *
+                             ((Dv + D + 63) / 64) < 1024)
+      chunk /= 2;
     while (chunk > 0 && (bound + chunk - 1) / chunk * n_seqs * rec > (1L << 31))
       chunk *= 2;                             // keep the scratch under 2 GiB
     const long wgs = (long)n_seqs * H * ((Dv + 63) / 64);
