@@ -87,7 +87,8 @@ XLLM_DEV void dr_gates(const DRArgs<T>& A, long row, int h, float* g,
 //         ([s*max_chunks + c][h][D][Dv + D])
 // mode 2: the same tokens from the state the scan left in the record's first
 //         Dv columns; outputs written, nothing stored
-template <typename T, int CPT>
+// NOOUT: a launch of mode 1 only; the read-out sums are not formed at all.
+template <typename T, int CPT, bool NOOUT>
 __global__ void __launch_bounds__(256) delta_rule_kernel(
     float* __restrict__ out, DRArgs<T> A, float* __restrict__ state,
     const int* __restrict__ slots, const int* __restrict__ cu_q,
@@ -212,7 +213,7 @@ __global__ void __launch_bounds__(256) delta_rule_kernel(
 #pragma unroll
           for (int c = 0; c < CPT; ++c) {
             ak[c] += S[m][c] * kk;
-            aq[c] += S[m][c] * qq;
+            if (!NOOUT) aq[c] += S[m][c] * qq;
           }
         }
       }
@@ -220,7 +221,7 @@ __global__ void __launch_bounds__(256) delta_rule_kernel(
 #pragma unroll
       for (int c = 0; c < CPT; ++c) {
         const float a = dr_row16_sum(ak[c]) * kscale;
-        const float cq = dr_row16_sum(aq[c]) * qscale;
+        const float cq = NOOUT ? 0.f : dr_row16_sum(aq[c]) * qscale;
         const float u = beta * (vs[tt * VS + j * CPT + c] - g * a);
         uk[c] = u * kscale;
         ak[c] = g * cq + kq * u;          // the token's output column
@@ -234,7 +235,7 @@ __global__ void __launch_bounds__(256) delta_rule_kernel(
           for (int c = 0; c < CPT; ++c) S[m][c] = g * S[m][c] + kk * uk[c];
         }
       }
-      if (mode != 1 && r == 0) {
+      if (!NOOUT && mode != 1 && r == 0) {
         float* op = out + ((long)(tb + tt) * heads + h) * Dv + col;
 #pragma unroll
         for (int c = 0; c < CPT; ++c)
@@ -264,73 +265,98 @@ __global__ void __launch_bounds__(256) delta_rule_kernel(
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float dr_f32x4;
 
 // S <- M_c S + N_c over the pieces of a sequence, for 16 columns of one head.
-// S sits in LDS as [rows][16]; a wave owns every fourth 16-row tile of the
-// result. v_mfma_f32_16x16x4_f32: lane l gives A[l & 15][l >> 4] and
-// B[l >> 4][l & 15] and holds C[(l >> 4) * 4 + r][l & 15]. Within a block of
-// 16 inner indices lane group g takes the indices 4g..4g+3 (one 16 B load of
-// its M row), the same permutation on both operands. The record's first Dv
-// columns (N) are overwritten with the state before the piece.
-__global__ void __launch_bounds__(256) delta_rule_scan_kernel(
+// S sits in LDS as [rows][16]; wave w owns the 16-row tile w of the result
+// (the workgroup has one wave per tile). v_mfma_f32_16x16x4_f32: lane l gives
+// A[l & 15][l >> 4] and B[l >> 4][l & 15] and holds C[(l >> 4) * 4 + r]
+// [l & 15]. Within a block of 16 inner indices lane group g takes the indices
+// 4g..4g+3 (one 16 B load of its M row), the same permutation on both
+// operands. A wave's M rows and N tile of the NEXT piece are loaded into
+// registers while the current piece multiplies (KB <= 8). The record's first
+// Dv columns (N) are overwritten with the state before the piece.
+template <int KB>                         // D <= 16 * KB
+__global__ void __launch_bounds__(64 * KB) delta_rule_scan_kernel(
     float* __restrict__ ws, float* __restrict__ state,
     const int* __restrict__ slots, const int* __restrict__ cu_q,
     const int* __restrict__ ctx_lens, int heads, int D, int Dv, int chunk,
     int max_chunks) {
   extern __shared__ float Sl[];           // [Dp][16]
+  constexpr bool PF = KB <= 8;
   const int s = blockIdx.x, h = blockIdx.y, col0 = blockIdx.z * 16;
-  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, it = tid >> 6;
+  const int nthr = blockDim.x;
   const int n = lane & 15, g = lane >> 4;
   const int E = Dv + D;
   const int qlen = cu_q[s + 1] - cu_q[s];
-  const int n_chunks = (qlen + chunk - 1) / chunk;
+  const int n_chunks = min((qlen + chunk - 1) / chunk, max_chunks);
   const int slot = slots[s];
   const int n_tiles = (D + 15) >> 4, Dp = n_tiles << 4;
   const bool col_ok = col0 + n < Dv;
   const bool from_slot = slot >= 0 && ctx_lens[s] > 0;
   float* sst = state + (((long)max(slot, 0) * heads + h) * D) * (long)Dv;
-  for (int idx = tid; idx < Dp * 16; idx += 256) {
+  for (int idx = tid; idx < Dp * 16; idx += nthr) {
     const int i = idx >> 4, jj = idx & 15;
     Sl[idx] = (from_slot && i < D && col0 + jj < Dv)
         ? sst[(long)i * Dv + col0 + jj] : 0.f;
   }
   __syncthreads();
   const bool fast = (D & 15) == 0 && (E & 3) == 0 && (Dv & 3) == 0;
-  constexpr int MAXT = 4;                 // D <= 256: 16 tiles over 4 waves
-  for (int c = 0; c < n_chunks; ++c) {
-    float* rec = ws + ((((long)s * max_chunks + c) * heads + h) * D) * (long)E;
-    dr_f32x4 acc[MAXT];
+  const int ia = it * 16 + n;             // this lane's M row
+  auto rec_of = [&](int c) {
+    return ws + ((((long)s * max_chunks + c) * heads + h) * D) * (long)E;
+  };
+  auto load = [&](const float* rec, float4 (&m4)[KB], float (&n4)[4]) {
+    const float* mrow = rec + (long)min(ia, D - 1) * E + Dv;
 #pragma unroll
-    for (int tt = 0; tt < MAXT; ++tt) {
-      const int it = wv + 4 * tt;
-      acc[tt] = dr_f32x4{0.f, 0.f, 0.f, 0.f};
-      if (it >= n_tiles) continue;        // uniform per wave
-#pragma unroll
-      for (int rr = 0; rr < 4; ++rr) {
-        const int i = it * 16 + 4 * g + rr;
-        if (i < D && col_ok) acc[tt][rr] = rec[(long)i * E + col0 + n];
-      }
-      const int ia = it * 16 + n;
-      const float* mrow = rec + (long)min(ia, D - 1) * E + Dv;
-      for (int kb = 0; kb < D; kb += 16) {
-        float a4[4];
+    for (int kbi = 0; kbi < KB; ++kbi) {
+      const int k0 = kbi * 16 + 4 * g;
+      m4[kbi] = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (kbi * 16 < D && it < n_tiles) {
         if (fast) {
-          const float4 x = *reinterpret_cast<const float4*>(mrow + kb + 4 * g);
-          a4[0] = x.x; a4[1] = x.y; a4[2] = x.z; a4[3] = x.w;
-        } else {
-#pragma unroll
-          for (int q4 = 0; q4 < 4; ++q4) {
-            const int ka = kb + 4 * g + q4;
-            a4[q4] = (ia < D && ka < D) ? mrow[ka] : 0.f;
-          }
-        }
-#pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4) {
-          const int kk = kb + 4 * g + q4;            // < Dp
-          acc[tt] = __builtin_amdgcn_mfma_f32_16x16x4f32(
-              a4[q4], Sl[kk * 16 + n], acc[tt], 0, 0, 0);
+          m4[kbi] = *reinterpret_cast<const float4*>(mrow + k0);
+        } else if (ia < D) {
+          if (k0 < D) m4[kbi].x = mrow[k0];
+          if (k0 + 1 < D) m4[kbi].y = mrow[k0 + 1];
+          if (k0 + 2 < D) m4[kbi].z = mrow[k0 + 2];
+          if (k0 + 3 < D) m4[kbi].w = mrow[k0 + 3];
         }
       }
-      // the state before this piece takes N's place (same thread, same
-      // elements it has just read)
+    }
+#pragma unroll
+    for (int rr = 0; rr < 4; ++rr) {
+      const int i = it * 16 + 4 * g + rr;
+      n4[rr] = (i < D && col_ok) ? rec[(long)i * E + col0 + n] : 0.f;
+    }
+  };
+  float4 mc[KB], mn[KB];               // mn unused without prefetch
+  float nc[4], nn[4];
+  if constexpr (PF) {
+    if (n_chunks > 0) load(rec_of(0), mc, nc);
+  }
+  for (int c = 0; c < n_chunks; ++c) {
+    float* rec = rec_of(c);
+    if constexpr (PF) {
+      if (c + 1 < n_chunks) load(rec_of(c + 1), mn, nn);
+    } else {
+      load(rec, mc, nc);
+    }
+    dr_f32x4 acc = {nc[0], nc[1], nc[2], nc[3]};
+    if (it < n_tiles) {                   // uniform per wave
+#pragma unroll
+      for (int kbi = 0; kbi < KB; ++kbi) {
+        if (kbi * 16 < D) {
+          const int kk = kbi * 16 + 4 * g;            // kk + 3 < Dp
+          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(
+              mc[kbi].x, Sl[kk * 16 + n], acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(
+              mc[kbi].y, Sl[(kk + 1) * 16 + n], acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(
+              mc[kbi].z, Sl[(kk + 2) * 16 + n], acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(
+              mc[kbi].w, Sl[(kk + 3) * 16 + n], acc, 0, 0, 0);
+        }
+      }
+      // the state before this piece takes N's place (this thread has read
+      // exactly these elements already)
 #pragma unroll
       for (int rr = 0; rr < 4; ++rr) {
         const int i = it * 16 + 4 * g + rr;
@@ -338,20 +364,23 @@ __global__ void __launch_bounds__(256) delta_rule_scan_kernel(
       }
     }
     __syncthreads();                      // every wave is done reading Sl
-#pragma unroll
-    for (int tt = 0; tt < MAXT; ++tt) {
-      const int it = wv + 4 * tt;
-      if (it >= n_tiles) continue;
+    if (it < n_tiles) {
 #pragma unroll
       for (int rr = 0; rr < 4; ++rr) {
         const int i = it * 16 + 4 * g + rr;
-        Sl[i * 16 + n] = (i < D && col_ok) ? acc[tt][rr] : 0.f;
+        Sl[i * 16 + n] = (i < D && col_ok) ? acc[rr] : 0.f;
       }
     }
     __syncthreads();
+    if constexpr (PF) {
+#pragma unroll
+      for (int kbi = 0; kbi < KB; ++kbi) mc[kbi] = mn[kbi];
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr) nc[rr] = nn[rr];
+    }
   }
   if (slot >= 0)
-    for (int idx = tid; idx < Dp * 16; idx += 256) {
+    for (int idx = tid; idx < Dp * 16; idx += nthr) {
       const int i = idx >> 4, jj = idx & 15;
       if (i < D && col0 + jj < Dv) sst[(long)i * Dv + col0 + jj] = Sl[idx];
     }
@@ -465,22 +494,27 @@ void launch_delta_rule_cpt(float* out, const DRArgs<T>& A, float* state,
                      sizeof(float);
   const int vz = (Dv + VS - 1) / VS;
   if (ws == nullptr || max_chunks <= 1) {
-    hipLaunchKernelGGL((delta_rule_kernel<T, CPT>), dim3(n_seqs, A.heads, vz),
-                       dim3(256), lds, st, out, A, state, slots, cu_q,
-                       ctx_lens, 0, 0, 1, nullptr);
+    hipLaunchKernelGGL((delta_rule_kernel<T, CPT, false>),
+                       dim3(n_seqs, A.heads, vz), dim3(256), lds, st, out, A,
+                       state, slots, cu_q, ctx_lens, 0, 0, 1, nullptr);
     return;
   }
   const int vz1 = (Dv + D + VS - 1) / VS;
-  hipLaunchKernelGGL((delta_rule_kernel<T, CPT>),
+  hipLaunchKernelGGL((delta_rule_kernel<T, CPT, true>),
                      dim3(n_seqs * max_chunks, A.heads, vz1), dim3(256), lds,
                      st, out, A, state, slots, cu_q, ctx_lens, 1, chunk,
                      max_chunks, ws);
-  const int Dp = ((D + 15) >> 4) << 4;
-  hipLaunchKernelGGL(delta_rule_scan_kernel,
-                     dim3(n_seqs, A.heads, (Dv + 15) / 16), dim3(256),
-                     (size_t)Dp * 16 * sizeof(float), st, ws, state, slots,
-                     cu_q, ctx_lens, A.heads, D, Dv, chunk, max_chunks);
-  hipLaunchKernelGGL((delta_rule_kernel<T, CPT>),
+  const int n_tiles = (D + 15) >> 4, Dp = n_tiles << 4;
+  const dim3 sgrid(n_seqs, A.heads, (Dv + 15) / 16);
+#define DR_SCAN(KB)                                                           \
+  hipLaunchKernelGGL(delta_rule_scan_kernel<KB>, sgrid, dim3(64 * KB),        \
+                     (size_t)Dp * 16 * sizeof(float), st, ws, state, slots,   \
+                     cu_q, ctx_lens, A.heads, D, Dv, chunk, max_chunks)
+  if (n_tiles <= 4) DR_SCAN(4);
+  else if (n_tiles <= 8) DR_SCAN(8);
+  else DR_SCAN(16);
+#undef DR_SCAN
+  hipLaunchKernelGGL((delta_rule_kernel<T, CPT, false>),
                      dim3(n_seqs * max_chunks, A.heads, vz), dim3(256), lds,
                      st, out, A, state, slots, cu_q, ctx_lens, 2, chunk,
                      max_chunks, ws);
