@@ -21,7 +21,8 @@ def _free_port():
 
 
 @pytest.mark.timeout(180)
-@pytest.mark.parametrize("model", ["llama-tiny", "dunusun-tiny"])
+@pytest.mark.parametrize("model", ["llama-tiny", "dunusun-tiny",
+                                   "tosipel-tiny"])
 def test_master_and_worker_cli(model):
     http_port, rpc_port, reg_port = _free_port(), _free_port(), _free_port()
     env = dict(os.environ)
