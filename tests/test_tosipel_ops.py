@@ -286,6 +286,50 @@ def test_batch_of_unequal_requests_on_scattered_pages(target, H, G, D, Dv,
     _close(out2, out[last].cpu(), target, "decode rows", 3)
 
 
+# ------------------------------------------- latent attention, no positions
+@pytest.mark.parametrize("target", TARGETS)
+@pytest.mark.parametrize("H,r", [(2, 12), (4, 64), (3, 40), (16, 128)])
+def test_latent_rows_without_rotated_part(target, H, r):
+    """The cached row is the normed latent alone (no rotated tail). Queries
+    already folded through the key up-projection are scored against the
+    rows; a key far back, on a page's last row, stands out for one query."""
+    dev, dt = target
+    g = torch.Generator().manual_seed(H * r)
+    L, n = 200, 6                          # context rows, then a portion of 6
+    raw = _rnd(g, L, r, dtype=dt)
+    w = 1.0 + 0.2 * torch.randn(r, generator=g)
+    nb = (L + BS - 1) // BS
+    order = torch.randperm(nb + 2, generator=g).tolist()[:nb]
+    cache = torch.zeros(nb + 2, BS, r, dtype=dt, device=dev)
+    slots = torch.tensor([order[p // BS] * BS + p % BS for p in range(L)])
+    none = torch.zeros(0, dtype=F64, device=dev)
+    hops.latent_kv_store(raw.to(dev), w.to(dev), 1e-5,
+                         torch.arange(L, device=dev), none, 1.0, 0, cache,
+                         slots.to(dev), r)
+    c = o_rms(raw.to(F64), 1e-5) * w.to(F64)
+    got_rows = cache.view(-1, r)[slots.to(dev)]
+    _close(got_rows, c, target, "rows", 2)
+    c = got_rows.cpu().to(F64)             # what the kernel reads
+    q = _rnd(g, n, H, r, dtype=dt, std=0.3)
+    far = 15                               # last row of the first page
+    q[n - 1] = (25.0 * c[far] / c[far].norm() ** 2).to(dt)
+    out = torch.empty(n, H, r, device=dev)
+    hops.latent_attn(q.to(dev), cache, _i32([order], dev), _i32([0, n], dev),
+                     _i32([L], dev), 0.8, r, out)
+    for i in range(n):
+        pos = L - n + i
+        for a in range(H):
+            want = o_attend(q[i, a].to(F64), c[:pos + 1], c[:pos + 1], 0.8)
+            _close(out[i, a], want, target, (i, a), 3)
+    assert float((out[n - 1, 0].cpu().to(F64) - c[far]).abs().max()) \
+        < 0.2 * float(c[far].abs().max())
+    # the last row once more as a decoded row
+    out2 = torch.empty(1, H, r, device=dev)
+    hops.latent_attn(q[n - 1:].to(dev), cache, _i32([order], dev), None,
+                     _i32([L], dev), 0.8, r, out2)
+    _close(out2[0], out[n - 1].cpu(), target, "decode row", 3)
+
+
 # ------------------------------------------------------------ the delta rule
 def _delta_inputs(g, T, H, G, D, Dv, dt):
     return (_rnd(g, T, G * D, dtype=dt), _rnd(g, T, G * D, dtype=dt),
