@@ -1,5 +1,8 @@
 """Hybrid-mixer ops: latent attention, decayed linear attention with a
-recurrent state, grouped RMS norms, gated residuals, routed experts.
+recurrent state, grouped RMS norms, gated residuals, routed experts;
+residual streams, short convolutions, gated recurrences, soft-capped and
+windowed paged attention; post-norm residual, whole-row q/k norm with
+rotate-half positions, the gated delta rule.
 
 Same policy as the rest of `ops`: on a GPU the HIP extension (`_ops_hybrid`)
 is the only path and its absence raises; on CPU the fp32 torch references in
