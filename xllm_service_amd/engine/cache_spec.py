@@ -4,7 +4,9 @@ A model may expose `cache_specs()` returning one spec per layer; the model
 runner allocates the tensors and hands layer i its entry of `kv_caches`:
 
   PagedKV          (k_cache, v_cache), [blocks, n_kv, block, head_dim] (the
-                   value cache has v_dim in place of head_dim when given)
+                   value cache has v_dim in place of head_dim when given;
+                   with values_are_keys there is one tensor, handed out as
+                   both members of the pair)
   PagedLatent      one tensor [blocks, block, width] (a shared row per token)
   RecurrentState   one fp32 tensor [state_slots, heads, dim, vdim]; a
                    sequence owns one slot for its whole life
@@ -27,14 +29,16 @@ class PagedKV:
     n_kv: int
     head_dim: int
     v_dim: Optional[int] = None          # None: values as wide as keys
+    values_are_keys: bool = False        # the layer reads its keys as values
 
     @property
     def value_dim(self) -> int:
         return self.head_dim if self.v_dim is None else self.v_dim
 
     def block_bytes(self, block_size: int, dtype_bytes: int) -> int:
-        return (self.n_kv * block_size * (self.head_dim + self.value_dim)
-                * dtype_bytes)
+        per_token = self.head_dim + (0 if self.values_are_keys
+                                     else self.value_dim)
+        return self.n_kv * block_size * per_token * dtype_bytes
 
 
 @dataclass(frozen=True)

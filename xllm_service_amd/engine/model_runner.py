@@ -47,6 +47,10 @@ class ModelRunner:
     def _allocate(self, spec):
         dtype, device = self.dtype, self.device
         slots = max(self.num_state_slots, 1)
+        if isinstance(spec, PagedKV) and spec.values_are_keys:
+            k = torch.zeros(self.num_blocks, spec.n_kv, BLOCK_SIZE,
+                            spec.head_dim, dtype=dtype, device=device)
+            return (k, k)
         if isinstance(spec, PagedKV):
             return tuple(
                 torch.zeros(self.num_blocks, spec.n_kv, BLOCK_SIZE, d,
@@ -85,7 +89,7 @@ class ModelRunner:
 
         def walk(spec, c):
             if isinstance(spec, PagedKV):
-                out.extend(c)
+                out.extend(c[:1] if spec.values_are_keys else c)
             elif isinstance(spec, PagedLatent):
                 out.append(c)
             elif isinstance(spec, CacheGroup):

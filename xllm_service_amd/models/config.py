@@ -10,7 +10,7 @@ from typing import List, Optional
 @dataclass
 class ModelConfig:
     name: str = "llama"
-    architecture: str = "llama"   # llama | opt | qwen2 | qwen2_vl | pugovik | dunusun | tosipel
+    architecture: str = "llama"   # llama | opt | qwen2 | qwen2_vl | pugovik | dunusun | tosipel | gararax
     vocab_size: int = 128256
     hidden_size: int = 4096
     intermediate_size: int = 14336
@@ -271,6 +271,74 @@ def tosipel_from_dict(d: dict, name: str = "tosipel",
         max_position=1 << 20, layers=layers, model_dir=model_dir)
 
 
+@dataclass
+class GararaxConfig(ModelConfig):
+    """Gararax: layers of grouped-head softmax attention in three kinds
+    (`attention`: pair-layout rotary with banded frequency scaling, unit RMS
+    norm of q and k, sliding window that also keeps the first tokens;
+    `attention_2`: no positions, values are the keys, a sink of score 0,
+    sigmoid output gate; `attention_3`: biased projections, half-layout
+    rotary, one score multiplier per head, every earlier key), RMS norms
+    before and after every sublayer, a scaled residual, dense PolyNorm or
+    routed-expert feed-forwards, a small per-layer token embedding added
+    after the feed-forward, a run of layers that repeats with the same
+    weights, and the embedding table as the head."""
+    layers: List[HybridLayerConfig] = field(default_factory=list)
+    residual_mult: float = 1.0
+    loop_start: int = 0
+    loop_stop: int = 0
+    loop_times: int = 1
+    side_dim: int = 0                   # per-layer token embedding (0: none)
+    model_dir: Optional[str] = None     # weights live here (None = random)
+
+    @property
+    def layer_runs(self) -> List[int]:
+        """Layer index of every layer run, in execution order (a looped
+        layer appears once per pass; each run owns its cache)."""
+        n = len(self.layers)
+        body = list(range(self.loop_start, self.loop_stop))
+        return (list(range(self.loop_start)) + body * self.loop_times
+                + list(range(self.loop_stop, n)))
+
+    @property
+    def has_recurrent_state(self) -> bool:
+        return False
+
+
+GARARAX_MIXERS = ("attention", "attention_2", "attention_3")
+
+
+def gararax_from_dict(d: dict, name: str = "gararax",
+                      model_dir: Optional[str] = None) -> GararaxConfig:
+    layers = [HybridLayerConfig(type=l["type"], mixer=dict(l["mixer"]),
+                                mlp=l.get("mlp"))
+              for l in d["layers"]]
+    for i, l in enumerate(layers):
+        if l.type not in GARARAX_MIXERS:
+            raise ValueError(f"layer {i}: unknown mixer type {l.type!r}")
+        if l.mlp is not None and l.mlp.get("kind") not in ("dense", "moe"):
+            raise ValueError(f"layer {i}: unknown feed-forward kind")
+        if l.type == "attention_2" and \
+                l.mixer.get("vdim", l.mixer["dim"]) != l.mixer["dim"]:
+            raise ValueError(f"layer {i}: values are keys, vdim must be dim")
+    lp = d.get("loop") or {}
+    start, stop = int(lp.get("start", 0)), int(lp.get("stop", 0))
+    times = int(lp.get("times", 1))
+    if not lp or stop <= start:
+        start = stop = 0
+        times = 1
+    if not (0 <= start <= stop <= len(layers)) or times < 1:
+        raise ValueError("loop: need 0 <= start <= stop <= layers, times >= 1")
+    return GararaxConfig(
+        name=name, architecture="gararax", vocab_size=int(d["vocab"]),
+        hidden_size=int(d["width"]), num_layers=len(layers),
+        rms_eps=float(d["norm"]["eps"]),
+        residual_mult=float(d.get("residual_mult", 1.0)),
+        loop_start=start, loop_stop=stop, loop_times=times,
+        side_dim=int((d.get("token_side") or {}).get("dim", 0)),
+        max_position=1 << 20, layers=layers, model_dir=model_dir)
+
+
 def load_model_dir(path: str) -> ModelConfig:
     """Read <path>/config.json and pick the config class by its
     `architecture` field."""
@@ -286,6 +354,9 @@ def load_model_dir(path: str) -> ModelConfig:
     if arch == "tosipel":
         return tosipel_from_dict(d, name=os.path.basename(
             os.path.normpath(path)) or "tosipel", model_dir=path)
+    if arch == "gararax":
+        return gararax_from_dict(d, name=os.path.basename(
+            os.path.normpath(path)) or "gararax", model_dir=path)
     raise ValueError(f"{path}: unsupported architecture "
                      f"{d.get('architecture')!r}")
 
@@ -425,6 +496,62 @@ PRESETS.update({
     # bench stacks at the width of real deployments (random weights)
     "tosipel-2k": _tosipel_preset("tosipel-2k", 2048, 8),
     "tosipel-4k": _tosipel_preset("tosipel-4k", 4096, 8),
+})
+
+
+def _gararax_preset(name, width, n_layers, vocab=32000, head=128, window=1024,
+                    keep_first=4, experts=16, top=2, identity=2, side=64,
+                    loop=None):
+    """Synthetic Gararax stacks for benchmarks: per group of four layers a
+    gated keys-as-values attention layer with a dense feed-forward, two
+    full-context biased layers and one windowed layer with routed experts
+    (plus identity experts and a shared expert)."""
+    heads = max(width // head, 1)
+    kv = max(heads // 4, 1)
+    n_all = experts + identity
+    groups = 4 if n_all % 4 == 0 and n_all >= 8 else 1
+    moe = dict(kind="moe", expert=dict(ff=width // 2),
+               router=dict(experts=experts, top=top, identity=identity,
+                           groups=dict(count=groups,
+                                       keep=max(groups // 2, 1))),
+               shared=dict(ff=width // 2))
+    dense = dict(kind="dense", ff=3 * width // 2)
+    layers = []
+    for i in range(n_layers):
+        k = i % 4
+        if k == 0:
+            layers.append(dict(type="attention_2", mlp=dense, mixer=dict(
+                heads=heads, kv_heads=kv, dim=head, vdim=head,
+                mask=dict(size=window, keep_first=keep_first),
+                scale=head ** -0.5)))
+        elif k == 3:
+            layers.append(dict(type="attention", mlp=moe, mixer=dict(
+                heads=heads, kv_heads=kv, dim=head, vdim=head,
+                mask=dict(size=window, keep_first=keep_first),
+                rot=dict(base=10000.0, dims=head // 2, scaling=dict(
+                    factor=8.0, low=1.0, high=4.0, original=8192)),
+                scale=1.0)))
+        else:
+            layers.append(dict(type="attention_3", mlp=moe, mixer=dict(
+                heads=heads, kv_heads=kv, dim=head, vdim=head,
+                rot=dict(base=10000.0, dims=head), scale=head ** -0.5)))
+    d = dict(architecture="Gararax", vocab=vocab, width=width, layers=layers,
+             norm=dict(eps=1e-6), residual_mult=0.5)
+    if side:
+        d["token_side"] = dict(dim=side)
+    if loop:
+        d["loop"] = dict(start=loop[0], stop=loop[1], times=loop[2])
+    return gararax_from_dict(d, name=name)
+
+
+PRESETS.update({
+    # CPU-test sized stack (layers 1..2 run twice)
+    "gararax-tiny": _gararax_preset("gararax-tiny", 64, 4, vocab=256, head=16,
+                                    window=20, keep_first=3, experts=6, top=2,
+                                    identity=2, side=8, loop=(1, 3, 2)),
+    # bench stacks at the width of real deployments (random weights)
+    "gararax-2k": _gararax_preset("gararax-2k", 2048, 8),
+    "gararax-4k": _gararax_preset("gararax-4k", 4096, 8),
 })
 
 

@@ -31,6 +31,13 @@ GatedDeltaRule         S <- g S; u = beta (v - S^T k); S <- S + k u^T;
                        o = S^T q with unit q, k after a short convolution and
                        SiLU; per-head scalar decay g; RMS norm per head, SiLU
                        gate.
+GroupedAttention       softmax attention with grouped key/value heads whose
+                       parts are all options: rotary positions in the pair or
+                       the half layout (plain or with banded frequency
+                       scaling), unit RMS norm of q and k per head after the
+                       turn, a sliding window that also keeps the first
+                       tokens, a sink of score 0, one score multiplier per
+                       head, keys read as values, element-wise sigmoid gate.
 
 All take the slice of a merged input projection that belongs to them and
 return the mixer output in the model dtype. Sizes and constants are
@@ -76,6 +83,28 @@ def scaled_rope_frequencies(rot: dict):
     ramp = torch.clamp((i - lo) / max(hi - lo, 0.001), 0.0, 1.0)
     f = f / factor * ramp + f * (1.0 - ramp)
     return f, 0.1 * math.log(factor) + 1.0
+
+
+def banded_rope_frequencies(rot: dict):
+    """Per-pair inverse frequencies (fp64) of a rotary config {base, dims,
+    scaling?}. With `scaling` = {factor, low, high, original} a frequency f
+    of wavelength l = 2 pi / f stays as it is for l < original / high,
+    becomes f / factor for l > original / low, and in between is the blend
+    (1 - s) f / factor + s f with s = (original / l - low) / (high - low)."""
+    dims, base = int(rot["dims"]), float(rot["base"])
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    f = base ** (-2.0 * i / dims)
+    sc = rot.get("scaling")
+    if not sc:
+        return f
+    factor, low, high = float(sc["factor"]), float(sc["low"]), \
+        float(sc["high"])
+    orig = float(sc["original"])
+    wl = 2.0 * math.pi / f
+    s = (orig / wl - low) / (high - low)
+    blend = (1.0 - s) * f / factor + s * f
+    return torch.where(wl < orig / high, f,
+                       torch.where(wl > orig / low, f / factor, blend))
 
 
 class LatentAttention(nn.Module):
@@ -519,4 +548,84 @@ class GatedDeltaRule(nn.Module):
         y = hops.gated_group_norm(o.view(T, b), self.out_norm, gate, self.eps,
                                   H, act_silu=True, gate_first=False,
                                   out_dtype=proj.dtype)
+        return F.linear(y, self.o_proj)
+
+
+class GroupedAttention(nn.Module):
+    """in_proj rows: [q: heads*dim | k: kv_heads*dim | v: kv_heads*vdim
+    (absent with values_are_keys) | g: heads*vdim (with gated)].
+
+    rot: {base, dims, scaling?} or None; rot_pairs: entries (2i, 2i+1) turn
+    together, else (i, i + dims/2). unit_norm: q and k are divided by their
+    root mean square per head after the turn. window 0 = every earlier key;
+    keep_first: the first keys stay visible beside the window. zero_sink: 1
+    joins the softmax denominator. head_scale: a learned score multiplier
+    per head. values_are_keys: the weighted sum runs over the cached keys.
+    gated: the heads' outputs are multiplied by sigmoid(g)."""
+
+    def __init__(self, width: int, heads: int, kv_heads: int, dim: int,
+                 vdim: int, rot: Optional[dict], rot_pairs: bool,
+                 scale: float, window: int, keep_first: int, norm_eps: float,
+                 dtype, *, unit_norm: bool = False, zero_sink: bool = False,
+                 head_scale: bool = False, values_are_keys: bool = False,
+                 gated: bool = False):
+        super().__init__()
+        if heads % kv_heads:
+            raise ValueError("heads must be a multiple of kv_heads")
+        if values_are_keys and vdim != dim:
+            raise ValueError("keys read as values: vdim must equal dim")
+        self.heads, self.kv_heads, self.dim, self.vdim = heads, kv_heads, \
+            dim, vdim
+        self.scale, self.eps = float(scale), norm_eps
+        self.window, self.keep_first = int(window), int(keep_first)
+        self.rot_pairs, self.unit_norm = bool(rot_pairs), bool(unit_norm)
+        self.values_are_keys, self.gated = values_are_keys, gated
+        self.rot_dims = int(rot["dims"]) if rot else 0
+        if self.rot_dims > dim or self.rot_dims % 2:
+            raise ValueError("rotary dims must be even and <= dim")
+        inv_freq = banded_rope_frequencies(rot) if self.rot_dims \
+            else torch.zeros(0, dtype=torch.float64)
+        self.register_buffer("inv_freq", inv_freq, persistent=False)
+        self.cq, self.ck = heads * dim, kv_heads * dim
+        self.cv = 0 if values_are_keys else kv_heads * vdim
+        self.g_width = heads * vdim if gated else 0
+        self.in_width = self.cq + self.ck + self.cv + self.g_width
+        f32 = dict(dtype=torch.float32)
+        if zero_sink:
+            self.register_buffer("sink", torch.zeros(heads, **f32),
+                                 persistent=False)
+        else:
+            self.sink = None
+        self.head_scale = nn.Parameter(torch.ones(heads, **f32)) \
+            if head_scale else None
+        self.o_proj = nn.Parameter(torch.empty(width, heads * vdim,
+                                               dtype=dtype))
+
+    def cache_spec(self):
+        return PagedKV(self.kv_heads, self.dim, self.vdim,
+                       values_are_keys=self.values_are_keys)
+
+    def forward(self, proj, positions, cache, meta: AttnMetadata, aux):
+        k_cache, v_cache = cache
+        T, cq, ck, cv = proj.shape[0], self.cq, self.ck, self.cv
+        H = self.heads
+        v_in = proj[:, cq + ck:cq + ck + cv] if cv else None
+        q = hops.rope_headnorm_store(
+            proj[:, :cq], proj[:, cq:cq + ck], v_in, positions, self.inv_freq,
+            self.rot_dims, self.rot_pairs, self.unit_norm, self.eps, H,
+            self.kv_heads, k_cache, v_cache, meta.slot_mapping)
+        o = torch.empty(T, H, self.vdim, dtype=torch.float32,
+                        device=proj.device)
+        for rows, cu_q, _, _, seq_lens, tables, _ in _halves(meta, aux):
+            hops.capped_attn(q[rows], k_cache, v_cache, tables, cu_q,
+                             seq_lens, H, self.scale, 0.0, o[rows],
+                             window=self.window, sink=self.sink,
+                             keep_first=self.keep_first,
+                             head_scale=self.head_scale)
+        o = o.view(T, H * self.vdim)
+        if self.gated:
+            y = hops.norm_sigmoid_gate(
+                o, None, proj[:, cq + ck + cv:self.in_width], 0.0, proj.dtype)
+        else:
+            y = o.to(proj.dtype)
         return F.linear(y, self.o_proj)

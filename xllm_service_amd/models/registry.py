@@ -27,11 +27,14 @@ def create_model(cfg: ModelConfig, dtype=torch.bfloat16):
     if cfg.architecture == "tosipel":
         from .tosipel import TosipelForCausalLM
         return TosipelForCausalLM(cfg, dtype=dtype)
+    if cfg.architecture == "gararax":
+        from .gararax import GararaxForCausalLM
+        return GararaxForCausalLM(cfg, dtype=dtype)
     raise ValueError(f"unknown architecture {cfg.architecture}")
 
 
 def required_extensions(cfg: ModelConfig):
     """In-tree HIP extension modules the model's GPU path loads."""
-    if cfg.architecture in ("pugovik", "dunusun", "tosipel"):
+    if cfg.architecture in ("pugovik", "dunusun", "tosipel", "gararax"):
         return ["_ops_hybrid"]
     return ["_ops"]

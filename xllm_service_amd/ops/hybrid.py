@@ -130,29 +130,40 @@ def decay_attn(q, k, v, decay, state, slots, cu_q, ctx_lens, out,
     return out
 
 
-def moe_route(h, w_router, top: int, n_groups: int, keep: int):
+def moe_route(h, w_router, top: int, n_groups: int, keep: int, *,
+              softmax: bool = False, correction=None, group_max: bool = False,
+              normalize: bool = False):
     """Router: fp32 logits h @ w_router^T (a true-fp32 library GEMM on the
-    GPU; h enters as stored, i.e. possibly bf16-rounded), then sigmoid
-    scores and the group-limited top-k selection kernel."""
+    GPU; h enters as stored, i.e. possibly bf16-rounded), then the scores
+    (sigmoid, or softmax over all experts) and the group-limited top-k
+    selection kernel. correction fp32 [experts] is added to the scores for
+    the choice only; group_max scores a group by its best expert instead of
+    its two best; normalize divides the chosen weights by their sum."""
     if h.is_cuda:
         T = h.shape[0]
         z = torch.matmul(h.float(), w_router.t())
         ids = torch.empty(T, top, dtype=torch.int32, device=h.device)
         wts = torch.empty(T, top, dtype=torch.float32, device=h.device)
-        _hyb().moe_route(ids, wts, z, top, n_groups, keep)
+        _hyb().moe_route(ids, wts, z, top, n_groups, keep, softmax,
+                         correction, group_max, normalize)
         return ids, wts
-    return ref.moe_route(h, w_router, top, n_groups, keep)
+    return ref.moe_route(h, w_router, top, n_groups, keep, softmax,
+                         correction, group_max, normalize)
 
 
-def moe_combine(y, rows, wts, tokens: int):
-    """fp32 [tokens, width] = sum_k wts[t, k] * y[rows[t, k]]."""
+def moe_combine(y, rows, wts, tokens: int, ident=None, extra=None):
+    """fp32 [tokens, width] = sum_k wts[t, k] * y[rows[t, k]] (+ extra[t]).
+    A negative row stands for the token's own input: ident[t]."""
     width = y.shape[-1]
     if y.is_cuda:
         out = torch.empty(tokens, width, dtype=torch.float32, device=y.device)
-        _hyb().moe_combine(out, y.view(-1, width), rows, wts)
+        _hyb().moe_combine(out, y.view(-1, width), rows, wts, ident, extra)
         return out
-    yy = y.reshape(-1, width).float()[rows.long()]          # [T, top, W]
-    return (yy * wts[:, :, None]).sum(1)
+    yy = y.reshape(-1, width).float()[rows.long().clamp(min=0)]   # [T,top,W]
+    if ident is not None:
+        yy = torch.where((rows < 0)[:, :, None], ident.float()[:, None, :], yy)
+    out = (yy * wts[:, :, None]).sum(1)
+    return out if extra is None else out + extra.float()
 
 
 # ---- residual streams, short convolutions, gated recurrences ---------------
@@ -270,28 +281,36 @@ def gated_group_norm(o, w, gate, eps: float, groups: int, *, act_silu: bool,
 
 def capped_attn(q, k_cache, v_cache, block_tables, cu_q, seq_lens,
                 heads: int, scale: float, cap: float, out, window: int = 0,
-                sink: Optional[torch.Tensor] = None):
+                sink: Optional[torch.Tensor] = None, keep_first: int = 0,
+                head_scale: Optional[torch.Tensor] = None):
     """out fp32 [T, heads, Dv] (written). cu_q None: decode rows. window > 0
-    limits a query to the last `window` keys (itself included); sink fp32
-    [heads] adds exp(sink_h) to the softmax denominator."""
+    limits a query to the last `window` keys (itself included) and, with
+    keep_first, the first keep_first keys of the sequence; sink fp32 [heads]
+    adds exp(sink_h) to the softmax denominator; head_scale fp32 [heads]
+    multiplies the scores of a head."""
+    if window <= 0:
+        keep_first = 0
     if q.is_cuda:
         _hyb().capped_attn(out, q, k_cache, v_cache, block_tables, cu_q,
-                           seq_lens, heads, scale, cap, window, sink)
+                           seq_lens, heads, scale, cap, window, sink,
+                           keep_first, head_scale)
         return out
     out.copy_(ref.capped_attn(q, k_cache, v_cache, block_tables, cu_q,
-                              seq_lens, heads, scale, cap, window, sink))
+                              seq_lens, heads, scale, cap, window, sink,
+                              keep_first, head_scale))
     return out
 
 
 # ---- post-norm residual, whole-row q/k norm, delta rule, GELU gate ----------
-def norm_residual_add_(x, y, w1, eps: float, out_dtype):
-    """x (fp32 [T, W], in place) += y / rms(y) * w1; returns the new x in
-    out_dtype (what the next sublayer multiplies)."""
+def norm_residual_add_(x, y, w1, eps: float, out_dtype, w_next=None):
+    """x (fp32 [T, W], in place) += y / rms(y) * w1 (y fp32 or model dtype).
+    Returns the new x in out_dtype, or with w_next the following sublayer's
+    normed input x / rms(x) * w_next from the same pass."""
     if x.is_cuda:
         h = torch.empty(x.shape, dtype=out_dtype, device=x.device)
-        _hyb().norm_residual_add(x, h, y, w1, eps)
+        _hyb().norm_residual_add(x, h, y, w1, eps, w_next)
         return h
-    return ref.norm_residual_add(x, y, w1, eps, out_dtype)
+    return ref.norm_residual_add(x, y, w1, eps, out_dtype, w_next)
 
 
 def rownorm_rope_store(q, k, v, q_w, k_w, eps: float, positions, inv_freq,
@@ -334,3 +353,42 @@ def gelu_tanh_mul(x):
         _hyb().gelu_tanh_mul(out, x)
         return out
     return ref.gelu_tanh_mul(x)
+
+
+# ---- rotary + unit head norm with paged store, PolyNorm, two-tensor gate ----
+def rope_headnorm_store(q, k, v, positions, inv_freq, rot_dims: int,
+                        pairs: bool, unit_norm: bool, eps: float, heads: int,
+                        kv_heads: int, k_cache, v_cache, slot_mapping):
+    """Rotary turn on the first rot_dims entries of every head of q [T,
+    heads*D] and k [T, kv_heads*D] (`pairs`: entries 2i / 2i+1, else i / i +
+    rot_dims/2), then with unit_norm each head divided by its root mean
+    square. Returns the new q as a contiguous tensor; k and v (None: the
+    values are the keys) go into the paged caches at the tokens' slots."""
+    if q.is_cuda:
+        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+        _hyb().rope_headnorm_store(out, q, k, v, positions, inv_freq,
+                                   rot_dims, pairs, unit_norm, eps, heads,
+                                   kv_heads, k_cache, v_cache, slot_mapping)
+        return out
+    return ref.rope_headnorm_store(q, k, v, positions, inv_freq, rot_dims,
+                                   pairs, unit_norm, eps, heads, kv_heads,
+                                   k_cache, v_cache, slot_mapping)
+
+
+def polynorm(z, coef, eps: float):
+    """coef[0] N(z) + coef[1] N(z^2) + coef[2] N(z^3) + coef[3] per row, N =
+    division by the root mean square of the row; fp32 inside."""
+    if z.is_cuda:
+        out = torch.empty(z.shape, dtype=z.dtype, device=z.device)
+        _hyb().polynorm(out, z, coef, eps)
+        return out
+    return ref.polynorm(z, coef, eps)
+
+
+def gelu_tanh_gate(g, u):
+    """gelu_tanh(g) * u, g and u [T, F] row views of one dtype."""
+    if g.is_cuda:
+        out = torch.empty(g.shape, dtype=g.dtype, device=g.device)
+        _hyb().gelu_tanh_gate(out, g, u)
+        return out
+    return ref.gelu_tanh_gate(g, u)

@@ -10,6 +10,7 @@ They are intentionally simple and readable, not fast.
 from __future__ import annotations
 
 import torch
+import torch.nn.functional as F
 
 
 def rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float) -> torch.Tensor:
@@ -283,23 +284,34 @@ def decay_linear_attn(q, k, v, decay, state, slots, cu_q, ctx_lens):
     return out
 
 
-def moe_route(h, w_router, top, n_groups, keep):
-    """Sigmoid-scored top-k routing with group limiting: experts form
-    n_groups equal neighbouring groups scored by the sum of their two
-    largest scores; only the best `keep` groups are eligible. Returns
-    (ids [T, top] int32, weights [T, top] fp32 = raw scores)."""
+def moe_route(h, w_router, top, n_groups, keep, softmax=False,
+              correction=None, group_max=False, normalize=False):
+    """Top-k routing with group limiting. Scores: sigmoid of the fp32 logits,
+    or their softmax over all experts. The choice is made on the scores plus
+    `correction` (when given); the weights are the plain scores of the
+    chosen, divided by their sum (+ 1e-20) with `normalize`. Experts form
+    n_groups equal neighbouring groups, scored by the sum of their two
+    largest choice scores (by the largest one with `group_max`); only the
+    best `keep` groups are eligible. Returns (ids [T, top] int32, weights
+    [T, top] fp32)."""
     z = h.float() @ w_router.float().T
-    s = torch.sigmoid(z)
+    s = torch.softmax(z, -1) if softmax else torch.sigmoid(z)
     T, E = s.shape
-    sm = s
+    sm = s if correction is None else s + correction.float()
     if n_groups > 1:
-        sg = s.view(T, n_groups, E // n_groups)
-        gs = sg.topk(min(2, E // n_groups), -1).values.sum(-1)
+        sg = sm.view(T, n_groups, E // n_groups)
+        if group_max:
+            gs = sg.max(-1).values
+        else:
+            gs = sg.topk(min(2, E // n_groups), -1).values.sum(-1)
         best = gs.topk(keep, -1).indices
         gm = torch.zeros_like(gs, dtype=torch.bool).scatter(1, best, True)
         sm = sg.masked_fill(~gm[:, :, None], float("-inf")).reshape(T, E)
     idx = sm.topk(top, -1).indices
-    return idx.to(torch.int32), s.gather(1, idx)
+    wts = s.gather(1, idx)
+    if normalize:
+        wts = wts / (wts.sum(-1, keepdim=True) + 1e-20)
+    return idx.to(torch.int32), wts
 
 
 def silu_mul(x):
@@ -453,12 +465,15 @@ def store_paged(x, cache, slot_mapping):
 
 
 def capped_attn(q, k_cache, v_cache, block_tables, cu_q, seq_lens, heads,
-                scale, cap, window=0, sink=None):
+                scale, cap, window=0, sink=None, keep_first=0,
+                head_scale=None):
     """Causal softmax attention of q [T, heads*D] over the paged caches
     [blocks, n_kv, block, D|Dv]; scores scale * q.k, then cap * tanh(. /
     cap) when cap > 0. window > 0: position i sees only the keys j with
     i - j < window. sink [heads]: exp(sink_h) joins the softmax denominator
-    (a key without a value). Returns fp32 [T, heads, Dv]."""
+    (a key without a value). keep_first: with a window, the keys j <
+    keep_first stay visible as well. head_scale [heads]: one more score
+    multiplier per head. Returns fp32 [T, heads, Dv]."""
     T = q.shape[0]
     nb, n_kv, bs, D = k_cache.shape
     Dv = v_cache.shape[3]
@@ -478,12 +493,17 @@ def capped_attn(q, k_cache, v_cache, block_tables, cu_q, seq_lens, heads,
         vv = vv.repeat_interleave(per, 0)
         qq = q[q0:q1].float().view(q1 - q0, heads, D)
         sc = torch.einsum("thd,hld->thl", qq, kk) * scale
+        if head_scale is not None:
+            sc = sc * head_scale.float()[None, :, None]
         if cap and cap > 0:
             sc = cap * torch.tanh(sc / cap)
         qpos = (ctx + torch.arange(q1 - q0))[:, None]
         mask = torch.arange(L)[None, :] > qpos
         if window and window > 0:
-            mask = mask | (torch.arange(L)[None, :] <= qpos - window)
+            gone = torch.arange(L)[None, :] <= qpos - window
+            if keep_first > 0:
+                gone = gone & (torch.arange(L)[None, :] >= keep_first)
+            mask = mask | gone
         sc = sc.masked_fill(mask[:, None, :], float("-inf"))
         if sink is None:
             p = torch.softmax(sc, -1)
@@ -500,11 +520,15 @@ def capped_attn(q, k_cache, v_cache, block_tables, cu_q, seq_lens, heads,
 # Post-norm residual, whole-row query/key norm with rotate-half positions,
 # gated delta rule, GELU-gated feed-forward. fp32 throughout.
 # ---------------------------------------------------------------------------
-def norm_residual_add(x, y, w1, eps, out_dtype):
-    """x (fp32, in place) += y / rms(y) * w1; returns x in out_dtype."""
+def norm_residual_add(x, y, w1, eps, out_dtype, w_next=None):
+    """x (fp32, in place) += y / rms(y) * w1; returns x in out_dtype, or
+    with w_next the next sublayer's input x / rms(x) * w_next."""
     yf = y.float()
     x.add_(yf * torch.rsqrt(yf.pow(2).mean(-1, keepdim=True) + eps) * w1)
-    return x.to(out_dtype)
+    if w_next is None:
+        return x.to(out_dtype)
+    return (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+            * w_next).to(out_dtype)
 
 
 def rope_halves(x, positions, inv_freq, rot_dims):
@@ -581,3 +605,50 @@ def delta_rule(q, k, v, b, a, dt_bias, A_log, state, slots, cu_q, ctx_lens,
 def gelu_tanh_mul(x):
     """[..., 2F] -> gelu_tanh(x[..., :F]) * x[..., F:], dtype preserved."""
     return gelu_and_mul(x)
+
+
+# ---------------------------------------------------------------------------
+# Rotary turn + unit norm per head with paged store, PolyNorm, GELU gate of
+# two tensors. fp32 throughout.
+# ---------------------------------------------------------------------------
+def rope_headnorm_store(q, k, v, positions, inv_freq, rot_dims, pairs,
+                        unit_norm, eps, heads, kv_heads, k_cache, v_cache,
+                        slot_mapping):
+    """q [T, heads*D], k [T, kv_heads*D]: rotary turn on the first rot_dims
+    entries of every head (`pairs`: entries 2i and 2i+1 turn together, else
+    i and i + rot_dims/2), then with `unit_norm` every head is divided by
+    its root mean square. Returns the new q; k and v (when given) go to the
+    paged caches."""
+    T = q.shape[0]
+
+    def prep(z, n):
+        z = z.reshape(T, n, -1)
+        if rot_dims:
+            z = (rope_interleaved(z.float(), positions, inv_freq, 1.0,
+                                  rot_dims) if pairs
+                 else rope_halves(z, positions, inv_freq, rot_dims))
+        z = z.float()
+        if unit_norm:
+            z = z * torch.rsqrt(z.pow(2).mean(-1, keepdim=True) + eps)
+        return z.reshape(T, -1)
+    store_paged(prep(k, kv_heads).to(k.dtype), k_cache, slot_mapping)
+    if v is not None:
+        store_paged(v, v_cache, slot_mapping)
+    return prep(q, heads).to(q.dtype)
+
+
+def polynorm(z, coef, eps):
+    """c0 N(z) + c1 N(z^2) + c2 N(z^3) + c3 with N(u) = u / rms(u) over the
+    last axis; coef fp32 [4]. dtype preserved."""
+    zf = z.float()
+
+    def unit(u):
+        return u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps)
+    out = (coef[0] * unit(zf) + coef[1] * unit(zf * zf)
+           + coef[2] * unit(zf * zf * zf) + coef[3])
+    return out.to(z.dtype)
+
+
+def gelu_tanh_gate(g, u):
+    """gelu_tanh(g) * u for two tensors of one shape, dtype of g."""
+    return (F.gelu(g.float(), approximate="tanh") * u.float()).to(g.dtype)
