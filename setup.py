@@ -48,8 +48,9 @@ ext_modules = [
     ),
     # hybrid sequence mixers (latent attention, decayed and gated linear
     # recurrences, the gated delta rule, soft-capped / windowed paged attention,
-    # short convolutions), grouped and post norms, residual streams and routed
-    # experts; bf16 and fp32 activations
+    # short convolutions, rotary turns with head norms), grouped and post
+    # norms, PolyNorm, residual streams and routed experts; bf16 and fp32
+    # activations
     CUDAExtension(
         name="xllm_service_amd._ops_hybrid",
         sources=[
@@ -59,7 +60,7 @@ ext_modules = [
                       "streams.hip", "short_conv.hip",
                       "gated_recurrence.hip", "capped_attn.hip",
                       "capped_attn_mfma.hip", "rownorm_rope.hip",
-                      "delta_rule.hip")
+                      "delta_rule.hip", "rope_headnorm.hip")
         ],
         extra_compile_args={
             "cxx": ["-O3", "-std=c++17"],

@@ -22,9 +22,20 @@ void launch_gated_norm_residual(float*, const TY*, const TG*, const float*,
 template <typename T>
 void launch_norm_sigmoid_gate(T*, const float*, const float*, const T*, float,
                               int, int, long, int, hipStream_t);
+template <typename TY, typename T>
+void launch_norm_residual_add(float*, T*, const TY*, const float*, float, int,
+                              int, long, const float*, hipStream_t);
 template <typename T>
-void launch_norm_residual_add(float*, T*, const T*, const float*, float, int,
-                              int, long, hipStream_t);
+void launch_rope_headnorm_store(T*, const T*, const T*, const T*, long, long,
+                                long, const long*, const double*, int, int,
+                                int, float, int, int, int, int, int, T*, T*,
+                                const long*, int, hipStream_t);
+template <typename T>
+void launch_polynorm(T*, const T*, const float*, float, long, int, long,
+                     hipStream_t);
+template <typename T>
+void launch_gelu_tanh_gate(T*, const T*, const T*, long, int, long, long,
+                           hipStream_t);
 template <typename T>
 void launch_silu_mul(T*, const T*, long, int, hipStream_t);
 template <typename T>
@@ -63,10 +74,10 @@ void launch_decay_attn(float*, const T*, const T*, const T*, const float*,
                        int, int, long, long, long, int, int, float*,
                        hipStream_t);
 void launch_moe_route(int*, float*, const float*, int, int, int, int, int,
-                      hipStream_t);
+                      int, const float*, int, int, hipStream_t);
 template <typename T>
 void launch_moe_combine(float*, const T*, const int*, const float*, long, int,
-                        int, hipStream_t);
+                        int, const T*, long, const T*, long, hipStream_t);
 template <typename TO>
 void launch_streams_mix_norm(TO*, const float*, const float*, const float*,
                              const float*, float, int, int, int, hipStream_t);
@@ -105,12 +116,13 @@ void launch_capped_attn_mfma(float*, float*, float*, const unsigned short*,
                              const unsigned short*, const unsigned short*,
                              const int*, const int*, const int*, int, int, int,
                              int, int, int, int, int, float, float, long, int,
-                             int, const float*, hipStream_t);
+                             int, const float*, int, const float*,
+                             hipStream_t);
 template <typename T>
 void launch_capped_attn(float*, const T*, const T*, const T*, const int*,
                         const int*, const int*, int, int, int, int, int, int,
-                        int, int, float, float, long, int, const float*,
-                        hipStream_t);
+                        int, int, float, float, long, int, const float*, int,
+                        const float*, hipStream_t);
 }  // namespace hyb
 }  // namespace xllm
 
@@ -209,18 +221,95 @@ void norm_sigmoid_gate(Tensor out, Tensor o, c10::optional<Tensor> w,
     hy::launch_norm_sigmoid_gate<bf>(ptr<bf>(out), ptr<float>(o), wp, ptr<bf>(gate), eps, rows, n, gate.stride(0), gate_cols, cur());
 }
 
-// res fp32 [rows, width] += y / rms(y) * w1; h = the new res in y's type
-void norm_residual_add(Tensor res, Tensor h, Tensor y, Tensor w1, double eps) {
+// res fp32 [rows, width] += y / rms(y) * w1 (y fp32 or h's type); h = the new
+// res, or with w_next res / rms(res) * w_next
+void norm_residual_add(Tensor res, Tensor h, Tensor y, Tensor w1, double eps,
+                       c10::optional<Tensor> w_next) {
   CHK_F32C(res); CHK_ACT(h); CHK_ACT(y); CHK_F32C(w1);
   TORCH_CHECK(res.dim() == 2 && y.dim() == 2 && h.is_contiguous() &&
-              h.dtype() == y.dtype());
+              (h.dtype() == y.dtype() || is_f32(y)));
   const int rows = res.size(0), width = res.size(1);
   TORCH_CHECK(y.size(0) == rows && y.size(1) == width &&
               h.numel() == res.numel() && w1.numel() == width);
-  if (is_f32(y))
-    hy::launch_norm_residual_add<float>(ptr<float>(res), ptr<float>(h), ptr<float>(y), ptr<float>(w1), eps, rows, width, y.stride(0), cur());
+  const float* wn = nullptr;
+  if (w_next.has_value()) {
+    CHK_F32C(*w_next);
+    TORCH_CHECK(w_next->numel() == width);
+    wn = ptr<float>(*w_next);
+  }
+  if (is_f32(y) && is_f32(h))
+    hy::launch_norm_residual_add<float, float>(ptr<float>(res), ptr<float>(h), ptr<float>(y), ptr<float>(w1), eps, rows, width, y.stride(0), wn, cur());
+  else if (is_f32(y))
+    hy::launch_norm_residual_add<float, bf>(ptr<float>(res), ptr<bf>(h), ptr<float>(y), ptr<float>(w1), eps, rows, width, y.stride(0), wn, cur());
   else
-    hy::launch_norm_residual_add<bf>(ptr<float>(res), ptr<bf>(h), ptr<bf>(y), ptr<float>(w1), eps, rows, width, y.stride(0), cur());
+    hy::launch_norm_residual_add<bf, bf>(ptr<float>(res), ptr<bf>(h), ptr<bf>(y), ptr<float>(w1), eps, rows, width, y.stride(0), wn, cur());
+}
+
+// out [rows, F] contiguous; z row view of the same type; coef fp32 [4]
+void polynorm(Tensor out, Tensor z, Tensor coef, double eps) {
+  CHK_ACT(out); CHK_ACT(z); CHK_F32C(coef);
+  TORCH_CHECK(out.dim() == 2 && z.dim() == 2 && out.is_contiguous() &&
+              out.dtype() == z.dtype() && out.size(0) == z.size(0) &&
+              out.size(1) == z.size(1) && coef.numel() == 4);
+  const long rows = z.size(0);
+  const int F = z.size(1);
+  if (is_f32(z)) hy::launch_polynorm<float>(ptr<float>(out), ptr<float>(z), ptr<float>(coef), eps, rows, F, z.stride(0), cur());
+  else hy::launch_polynorm<bf>(ptr<bf>(out), ptr<bf>(z), ptr<float>(coef), eps, rows, F, z.stride(0), cur());
+}
+
+// out [rows, F] contiguous = gelu_tanh(g) * u; g, u row views
+void gelu_tanh_gate(Tensor out, Tensor g, Tensor u) {
+  CHK_ACT(out); CHK_ACT(g); CHK_ACT(u);
+  TORCH_CHECK(out.dim() == 2 && g.dim() == 2 && u.dim() == 2 &&
+              out.is_contiguous() && out.dtype() == g.dtype() &&
+              out.dtype() == u.dtype() && g.sizes() == out.sizes() &&
+              u.sizes() == out.sizes());
+  const long rows = out.size(0);
+  const int F = out.size(1);
+  if (is_f32(g)) hy::launch_gelu_tanh_gate<float>(ptr<float>(out), ptr<float>(g), ptr<float>(u), rows, F, g.stride(0), u.stride(0), cur());
+  else hy::launch_gelu_tanh_gate<bf>(ptr<bf>(out), ptr<bf>(g), ptr<bf>(u), rows, F, g.stride(0), u.stride(0), cur());
+}
+
+// q_out [T, H*D] contiguous; q/k/v row views of a projection (v absent: the
+// values are the keys); caches [blocks, n_kv, block, D | Dv]
+void rope_headnorm_store(Tensor q_out, Tensor q, Tensor k,
+                         c10::optional<Tensor> v, Tensor pos, Tensor inv_freq,
+                         long rot, bool pairs, bool unit, double eps,
+                         long heads, long n_kv, Tensor k_cache,
+                         Tensor v_cache, Tensor slot_mapping) {
+  CHK_ACT(q_out); CHK_ACT(q); CHK_ACT(k); CHK_I64C(pos);
+  CHK_I64C(slot_mapping); CHK_ACT(k_cache); CHK_ACT(v_cache);
+  TORCH_CHECK(q.dim() == 2 && k.dim() == 2 && q_out.is_contiguous() &&
+              k_cache.dim() == 4 && v_cache.dim() == 4 &&
+              k_cache.is_contiguous() && v_cache.is_contiguous());
+  TORCH_CHECK(q.dtype() == k.dtype() && q.dtype() == q_out.dtype() &&
+              q.dtype() == k_cache.dtype() && q.dtype() == v_cache.dtype());
+  const int T = q.size(0), D = k_cache.size(3), Dv = v_cache.size(3);
+  const int bs = k_cache.size(2);
+  TORCH_CHECK(heads >= 1 && n_kv >= 1 && D <= 64 * 8 &&
+              q.size(1) == heads * D && k.size(1) == n_kv * D &&
+              k.size(0) == T && q_out.numel() == q.numel() &&
+              k_cache.size(1) == n_kv && v_cache.size(1) == n_kv &&
+              v_cache.size(2) == bs && v_cache.size(0) == k_cache.size(0) &&
+              pos.numel() == T && slot_mapping.numel() == T,
+              "rope_headnorm_store: bad shapes");
+  TORCH_CHECK(rot >= 0 && rot % 2 == 0 && rot <= D &&
+              inv_freq.is_cuda() && inv_freq.dtype() == torch::kDouble &&
+              inv_freq.is_contiguous() && inv_freq.numel() == rot / 2);
+  const void* vp = nullptr;
+  long vs = 0;
+  if (v.has_value()) {
+    CHK_ACT(*v);
+    TORCH_CHECK(v->dim() == 2 && v->dtype() == q.dtype() &&
+                v->size(0) == T && v->size(1) == n_kv * Dv,
+                "rope_headnorm_store: bad value rows");
+    vp = v->data_ptr();
+    vs = v->stride(0);
+  }
+  if (is_f32(q))
+    hy::launch_rope_headnorm_store<float>(ptr<float>(q_out), ptr<float>(q), ptr<float>(k), (const float*)vp, q.stride(0), k.stride(0), vs, ptr<long>(pos), ptr<double>(inv_freq), rot, pairs, unit, eps, T, heads, n_kv, D, Dv, ptr<float>(k_cache), ptr<float>(v_cache), ptr<long>(slot_mapping), bs, cur());
+  else
+    hy::launch_rope_headnorm_store<bf>(ptr<bf>(q_out), ptr<bf>(q), ptr<bf>(k), (const bf*)vp, q.stride(0), k.stride(0), vs, ptr<long>(pos), ptr<double>(inv_freq), rot, pairs, unit, eps, T, heads, n_kv, D, Dv, ptr<bf>(k_cache), ptr<bf>(v_cache), ptr<long>(slot_mapping), bs, cur());
 }
 
 void gelu_tanh_mul(Tensor out, Tensor x) {
@@ -491,7 +580,8 @@ void decay_attn(Tensor out, Tensor q, Tensor k, Tensor v, Tensor decay,
 
 // z fp32 [T, E] router logits -> ids int32 [T, top], wts fp32 [T, top]
 void moe_route(Tensor ids, Tensor wts, Tensor z, long top, long n_groups,
-               long keep) {
+               long keep, bool softmax, c10::optional<Tensor> correction,
+               bool group_max, bool normalize) {
   CHK_I32C(ids); CHK_F32C(wts); CHK_F32C(z);
   TORCH_CHECK(z.dim() == 2);
   const int T = z.size(0), E = z.size(1);
@@ -500,22 +590,46 @@ void moe_route(Tensor ids, Tensor wts, Tensor z, long top, long n_groups,
               keep >= 1 && keep <= n_groups &&
               keep * (E / n_groups) >= top, "bad routing constants");
   TORCH_CHECK((2 * E + n_groups) * 4 <= 64 * 1024, "too many experts");
+  const float* corr = nullptr;
+  if (correction.has_value()) {
+    CHK_F32C(*correction);
+    TORCH_CHECK(correction->numel() == E);
+    corr = ptr<float>(*correction);
+  }
   hy::launch_moe_route(ptr<int>(ids), ptr<float>(wts), ptr<float>(z), T, E,
-                       top, n_groups, keep, cur());
+                       top, n_groups, keep, softmax, corr, group_max,
+                       normalize, cur());
 }
 
-// out fp32 [T, width]; y [R, width] contiguous; rows int32 [T, top] < R
-void moe_combine(Tensor out, Tensor y, Tensor rows, Tensor wts) {
+// out fp32 [T, width]; y [R, width] contiguous; rows int32 [T, top] < R, a
+// negative row reads ident [T, width] (0 without one); extra [T, width] is
+// added
+void moe_combine(Tensor out, Tensor y, Tensor rows, Tensor wts,
+                 c10::optional<Tensor> ident, c10::optional<Tensor> extra) {
   CHK_F32C(out); CHK_ACT(y); CHK_I32C(rows); CHK_F32C(wts);
   TORCH_CHECK(y.is_contiguous() && out.dim() == 2 && rows.dim() == 2);
   const long T = out.size(0);
   const int width = out.size(1), top = rows.size(1);
   TORCH_CHECK(rows.size(0) == T && wts.numel() == T * top &&
               y.size(-1) == width);
+  const void *ip = nullptr, *ep = nullptr;
+  long is = 0, es = 0;
+  if (ident.has_value()) {
+    CHK_ACT(*ident);
+    TORCH_CHECK(ident->dim() == 2 && ident->size(0) == T &&
+                ident->size(1) == width && ident->dtype() == y.dtype());
+    ip = ident->data_ptr(); is = ident->stride(0);
+  }
+  if (extra.has_value()) {
+    CHK_ACT(*extra);
+    TORCH_CHECK(extra->dim() == 2 && extra->size(0) == T &&
+                extra->size(1) == width && extra->dtype() == y.dtype());
+    ep = extra->data_ptr(); es = extra->stride(0);
+  }
   if (is_f32(y))
-    hy::launch_moe_combine<float>(ptr<float>(out), ptr<float>(y), ptr<int>(rows), ptr<float>(wts), T, width, top, cur());
+    hy::launch_moe_combine<float>(ptr<float>(out), ptr<float>(y), ptr<int>(rows), ptr<float>(wts), T, width, top, (const float*)ip, is, (const float*)ep, es, cur());
   else
-    hy::launch_moe_combine<bf>(ptr<float>(out), ptr<bf>(y), ptr<int>(rows), ptr<float>(wts), T, width, top, cur());
+    hy::launch_moe_combine<bf>(ptr<float>(out), ptr<bf>(y), ptr<int>(rows), ptr<float>(wts), T, width, top, (const bf*)ip, is, (const bf*)ep, es, cur());
 }
 
 // x fp32 [T, S, W]; out [T, W] = layernorm(sum_s w_in[s] x[:, s]) * g + b
@@ -820,7 +934,8 @@ void gated_group_norm(Tensor out, Tensor o, Tensor w, Tensor gate, double eps,
 void capped_attn(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
                  Tensor block_tables, c10::optional<Tensor> cu_q,
                  Tensor seq_lens, long heads, double scale, double cap,
-                 long window, c10::optional<Tensor> sink) {
+                 long window, c10::optional<Tensor> sink, long keep_first,
+                 c10::optional<Tensor> head_scale) {
   CHK_F32C(out); CHK_ACT(q); CHK_ACT(k_cache); CHK_ACT(v_cache);
   CHK_I32C(block_tables); CHK_I32C(seq_lens);
   TORCH_CHECK(q.dim() == 2 && k_cache.dim() == 4 && v_cache.dim() == 4 &&
@@ -851,6 +966,14 @@ void capped_attn(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
     TORCH_CHECK(sink->numel() == heads);
     sinkp = ptr<float>(*sink);
   }
+  TORCH_CHECK(keep_first >= 0 && keep_first < (1L << 30) &&
+              (keep_first == 0 || window > 0), "bad keep_first");
+  const float* hsp = nullptr;
+  if (head_scale.has_value()) {
+    CHK_F32C(*head_scale);
+    TORCH_CHECK(head_scale->numel() == heads);
+    hsp = ptr<float>(*head_scale);
+  }
   // bf16: MFMA kernel when the sizes fit one of its instantiations
   if (is_bf16(q) && hy::capped_attn_mfma_class(D, Dv) != 0 &&
       q.stride(0) % 8 == 0 &&
@@ -866,7 +989,9 @@ void capped_attn(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
       const int rows_wg = per <= 16 ? 16 : per <= 32 ? 32 : 64;
       const long wgs = (long)T * n_kv * ((per + rows_wg - 1) / rows_wg);
       long max_tiles = ((long)block_tables.size(1) * bs + 31) / 32;
-      if (window > 0) max_tiles = std::min<long>(max_tiles, (window + 31) / 32 + 1);
+      if (window > 0)
+        max_tiles = std::min<long>(
+            max_tiles, (window + 31) / 32 + 1 + (keep_first + 31) / 32);
       n_part = (int)std::min<long>(std::min<long>(32, (max_tiles + 1) / 2),
                                    std::max<long>(1, 1024 / wgs));
       n_part = std::max(n_part, 1);
@@ -883,14 +1008,14 @@ void capped_attn(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
         n_part > 1 ? ptr<float>(ws_ml) : nullptr, ptr<bf>(q), ptr<bf>(k_cache),
         ptr<bf>(v_cache), ptr<int>(block_tables), cu, ptr<int>(seq_lens), T,
         n_seqs, heads, n_kv, D, Dv, bs, block_tables.size(1), scale, cap,
-        q.stride(0), n_part, window, sinkp, cur());
+        q.stride(0), n_part, window, sinkp, keep_first, hsp, cur());
     return;
   }
   TORCH_CHECK((size_t)4 * D * 4 <= 64 * 1024, "query row too wide for LDS");
   if (is_f32(q))
-    hy::launch_capped_attn<float>(ptr<float>(out), ptr<float>(q), ptr<float>(k_cache), ptr<float>(v_cache), ptr<int>(block_tables), cu, ptr<int>(seq_lens), T, n_seqs, heads, n_kv, D, Dv, bs, block_tables.size(1), scale, cap, q.stride(0), window, sinkp, cur());
+    hy::launch_capped_attn<float>(ptr<float>(out), ptr<float>(q), ptr<float>(k_cache), ptr<float>(v_cache), ptr<int>(block_tables), cu, ptr<int>(seq_lens), T, n_seqs, heads, n_kv, D, Dv, bs, block_tables.size(1), scale, cap, q.stride(0), window, sinkp, keep_first, hsp, cur());
   else
-    hy::launch_capped_attn<bf>(ptr<float>(out), ptr<bf>(q), ptr<bf>(k_cache), ptr<bf>(v_cache), ptr<int>(block_tables), cu, ptr<int>(seq_lens), T, n_seqs, heads, n_kv, D, Dv, bs, block_tables.size(1), scale, cap, q.stride(0), window, sinkp, cur());
+    hy::launch_capped_attn<bf>(ptr<float>(out), ptr<bf>(q), ptr<bf>(k_cache), ptr<bf>(v_cache), ptr<int>(block_tables), cu, ptr<int>(seq_lens), T, n_seqs, heads, n_kv, D, Dv, bs, block_tables.size(1), scale, cap, q.stride(0), window, sinkp, keep_first, hsp, cur());
 }
 
 }  // namespace
@@ -920,4 +1045,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("gelu_tanh_mul", &gelu_tanh_mul);
   m.def("rownorm_rope_store", &rownorm_rope_store);
   m.def("delta_rule", &delta_rule);
+  m.def("rope_headnorm_store", &rope_headnorm_store);
+  m.def("polynorm", &polynorm);
+  m.def("gelu_tanh_gate", &gelu_tanh_gate);
 }

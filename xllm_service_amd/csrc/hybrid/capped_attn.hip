@@ -5,9 +5,10 @@
 //   s_ij = scale * (q_i . k_j);  s_ij <- cap * tanh(s_ij / cap);
 //   o_i  = sum_j softmax_j(s_ij) v_j        over keys j <= i
 //
-// Optional: a sliding window (only the keys with i - j < window are seen) and
-// a per-head sink, a learned score without key or value whose exponential
-// joins the softmax denominator.
+// Optional: a sliding window (only the keys with i - j < window are seen; with
+// keep_first the keys j < keep_first stay visible beside it), a per-head sink,
+// a score without key or value whose exponential joins the softmax
+// denominator, and one more score multiplier per head.
 //
 // Caches: keys [blocks, n_kv, block, D], values [blocks, n_kv, block, Dv].
 // Scores, softmax weights and the weighted sum are fp32 for both storage
@@ -30,7 +31,8 @@ __global__ void capped_attn_kernel(
     const int* __restrict__ block_tables, const int* __restrict__ cu_q,
     const int* __restrict__ seq_lens, int n_seqs, int heads, int n_kv, int D,
     int Dv, int block_size, int table_width, float scale, float cap,
-    long q_row_stride, int window, const float* __restrict__ sink) {
+    long q_row_stride, int window, const float* __restrict__ sink,
+    int keep_first, const float* __restrict__ head_scale) {
   extern __shared__ float smem[];
   const int t = blockIdx.x;
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
@@ -62,33 +64,40 @@ __global__ void capped_attn_kernel(
   const int kvh = h / (heads / n_kv);
   const int* table = block_tables + (long)s * table_width;
   const float inv_cap = cap > 0.f ? 1.0f / cap : 0.f;
+  const float hs = head_scale != nullptr ? head_scale[h] : 1.0f;
   float m = -INFINITY, l = 0.f;
   float acc[CA_MAX_ACC];
 #pragma unroll
   for (int i = 0; i < CA_MAX_ACC; ++i) acc[i] = 0.f;
   const int n_acc = (Dv + 63) >> 6;
 
+  // two key ranges: the kept first keys that lie before the window, then
+  // the window itself (all keys without one)
   const int k_first = window > 0 ? max(0, n_keys - window) : 0;
-  for (int k0 = k_first; k0 < n_keys; k0 += 64) {
+  const int kept = window > 0 ? min(keep_first, k_first) : 0;
+  for (int seg = 0; seg < 2; ++seg) {
+  const int seg_lo = seg == 0 ? 0 : k_first;
+  const int seg_hi = seg == 0 ? kept : n_keys;
+  for (int k0 = seg_lo; k0 < seg_hi; k0 += 64) {
     const int key = k0 + lane;
     float sc = -INFINITY;
-    if (key < n_keys) {
+    if (key < seg_hi) {
       const long blk = table[key / block_size];
       const T* krow = k_cache +
           ((blk * n_kv + kvh) * block_size + key % block_size) * (long)D;
       float d = 0.f;
       for (int i = 0; i < D; ++i) d += qs[i] * IO<T>::ld(krow + i);
-      sc = d * scale;
+      sc = d * scale * hs;
       if (cap > 0.f) sc = cap * tanhf(sc * inv_cap);
     }
     const float m_new = fmaxf(m, wave_reduce_max(sc));
     const float alpha = expf(m - m_new);         // m=-inf first: exp(-inf)=0
-    const float p = (key < n_keys) ? expf(sc - m_new) : 0.f;
+    const float p = (key < seg_hi) ? expf(sc - m_new) : 0.f;
     l = l * alpha + wave_reduce_sum(p);
     m = m_new;
 #pragma unroll
     for (int i = 0; i < CA_MAX_ACC; ++i) acc[i] *= alpha;
-    const int nk = min(64, n_keys - k0);
+    const int nk = min(64, seg_hi - k0);
     for (int j = 0; j < nk; ++j) {
       const float pj = __shfl(p, j, 64);
       const int kj = k0 + j;
@@ -101,6 +110,7 @@ __global__ void capped_attn_kernel(
         if (i < n_acc && c < Dv) acc[i] += pj * IO<T>::ld(vrow + c);
       }
     }
+  }
   }
   if (sink != nullptr) {                  // a key without a value
     const float sk = sink[h];
@@ -126,7 +136,8 @@ void launch_capped_attn(float* out, const T* q, const T* k_cache,
                         int n_seqs, int heads, int n_kv, int D, int Dv,
                         int block_size, int table_width, float scale,
                         float cap, long q_row_stride, int window,
-                        const float* sink, hipStream_t st) {
+                        const float* sink, int keep_first,
+                        const float* head_scale, hipStream_t st) {
   if (tokens == 0) return;
   const int nw = heads < 4 ? heads : 4;
   dim3 grid(tokens, (heads + nw - 1) / nw);
@@ -134,14 +145,14 @@ void launch_capped_attn(float* out, const T* q, const T* k_cache,
                      (size_t)nw * D * sizeof(float), st, out, q, k_cache,
                      v_cache, block_tables, cu_q, seq_lens, n_seqs, heads,
                      n_kv, D, Dv, block_size, table_width, scale, cap,
-                     q_row_stride, window, sink);
+                     q_row_stride, window, sink, keep_first, head_scale);
 }
 
 #define INST_CA(T)                                                          \
   template void launch_capped_attn<T>(                                      \
       float*, const T*, const T*, const T*, const int*, const int*,         \
       const int*, int, int, int, int, int, int, int, int, float, float,     \
-      long, int, const float*, hipStream_t);
+      long, int, const float*, int, const float*, hipStream_t);
 INST_CA(float)
 INST_CA(unsigned short)
 

@@ -33,9 +33,12 @@
 // Decode splits the context over `n_part` workgroups per (token, key/value
 // head); partial (acc, max, sum) triples are merged by a second small kernel.
 //
-// Sliding window: a row sees the keys [limit - window, limit); the tile loop
-// starts at the first tile any row of the workgroup needs. Sink: exp(sink_h)
-// joins the denominator once, at the end (or in the merge kernel).
+// Sliding window: a row sees the keys [limit - window, limit) and, with
+// keep_first, the keys [0, keep_first) as well; the tile loop runs over the
+// leading tiles that hold kept keys and then from the first tile any row of
+// the workgroup needs (one list of tiles, split evenly over the context
+// partitions). Sink: exp(sink_h) joins the denominator once, at the end (or
+// in the merge kernel). head_scale: one more score multiplier per head.
 //
 // Fragment layouts of __builtin_amdgcn_mfma_f32_16x16x32_bf16 (lane l):
 //   A[l&15][(l>>4)*8 + j], B[(l>>4)*8 + j][l&15], C[(l>>4)*4 + r][l&15].
@@ -73,7 +76,8 @@ __global__ void __launch_bounds__(256) capped_attn_mfma_kernel(
     const int* __restrict__ block_tables, const int* __restrict__ cu_q,
     const int* __restrict__ seq_lens, int n_seqs, int heads, int n_kv, int D,
     int Dv, int block_size, int table_width, float scale, float cap,
-    long q_stride, int n_part, int window, const float* __restrict__ sink) {
+    long q_stride, int n_part, int window, const float* __restrict__ sink,
+    int keep_first, const float* __restrict__ head_scale) {
   extern __shared__ unsigned short cm_lds[];      // [key image | value image]
   __shared__ int tbl[512];                        // block ids of this key range
   constexpr int RT = 4 / CS;                      // row tiles per workgroup
@@ -117,9 +121,16 @@ __global__ void __launch_bounds__(256) capped_attn_mfma_kernel(
   // first key the earliest row of this workgroup sees
   const int kmin = window > 0 ? max(0, ctx + row0 / per + 1 - window) : 0;
   const int t_first = kmin / CM_KT;
-  const int tpp = (n_tiles - t_first + n_part - 1) / n_part;
-  const int t_begin = t_first + blockIdx.y * tpp;
-  const int t_end = min(n_tiles, t_begin + tpp);
+  // tile list: [0, t_keep) then [t_first, n_tiles)
+  const int t_keep = (window > 0 && keep_first > 0)
+      ? min((min(keep_first, kmax) + CM_KT - 1) / CM_KT, t_first) : 0;
+  const int n_list = t_keep + n_tiles - t_first;
+  const int tpp = (n_list + n_part - 1) / n_part;
+  const int i_begin = blockIdx.y * tpp;
+  const int i_end = min(n_list, i_begin + tpp);
+  auto tile_at = [&](int i) { return i < t_keep ? i : t_first + (i - t_keep); };
+  const int t_begin = tile_at(i_begin);
+  const int t_end = i_end > i_begin ? tile_at(i_end - 1) + 1 : t_begin;
   const int* table = block_tables + (long)s * table_width;
 
   // ---- this lane's row -----------------------------------------------------
@@ -146,12 +157,14 @@ __global__ void __launch_bounds__(256) capped_attn_mfma_kernel(
   for (int i = 0; i < NBL * 4; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
   const float inv_cap = cap > 0.f ? 1.0f / cap : 0.f;
+  const float hs = head_scale != nullptr ? head_scale[head] : 1.0f;
 
   constexpr int CHK = Dp >> 3, CHV = Dvp >> 3;       // 16 B chunks per row
-  // block ids of the keys [t_begin*32, t_end*32) into LDS (when they fit)
+  // block ids of the keys [t_begin*32, t_end*32) into LDS (when they fit;
+  // the range spans the gap between kept and window tiles, if there is one)
   const int blk0 = t_begin * CM_KT / block_size;
   const int nblk = (min(t_end * CM_KT, kmax) + block_size - 1) / block_size - blk0;
-  const bool tbl_ok = nblk <= 512;
+  const bool tbl_ok = nblk <= 512 && nblk > 0;
   if (tbl_ok)
     for (int i = tid; i < nblk; i += 256) tbl[i] = table[blk0 + i];
   __syncthreads();
@@ -184,14 +197,15 @@ __global__ void __launch_bounds__(256) capped_attn_mfma_kernel(
     }
   };
   cm_u16x8 prek[PF ? NPK : 1], prev[PF ? NPV : 1];
-  if (PF && t_begin < t_end) {
+  if (PF && i_begin < i_end) {
 #pragma unroll
     for (int i = 0; i < NPK; ++i) prek[i] = fetch(k_cache, D, CHK, t_begin, i);
 #pragma unroll
     for (int i = 0; i < NPV; ++i) prev[i] = fetch(v_cache, Dv, CHV, t_begin, i);
   }
 
-  for (int t = t_begin; t < t_end; ++t) {
+  for (int it = i_begin; it < i_end; ++it) {
+    const int t = tile_at(it);
     const int k0 = t * CM_KT;
     __syncthreads();
     if (PF) {
@@ -206,11 +220,12 @@ __global__ void __launch_bounds__(256) capped_attn_mfma_kernel(
       for (int i = 0; i < NPV; ++i) put(vt, CHV, i, fetch(v_cache, Dv, CHV, t, i));
     }
     __syncthreads();
-    if (PF && t + 1 < t_end) {          // next tile flies during the compute
+    if (PF && it + 1 < i_end) {         // next tile flies during the compute
+      const int tn = tile_at(it + 1);
 #pragma unroll
-      for (int i = 0; i < NPK; ++i) prek[i] = fetch(k_cache, D, CHK, t + 1, i);
+      for (int i = 0; i < NPK; ++i) prek[i] = fetch(k_cache, D, CHK, tn, i);
 #pragma unroll
-      for (int i = 0; i < NPV; ++i) prev[i] = fetch(v_cache, Dv, CHV, t + 1, i);
+      for (int i = 0; i < NPV; ++i) prev[i] = fetch(v_cache, Dv, CHV, tn, i);
     }
     if (!wave_on) continue;
     // ---- scores ------------------------------------------------------------
@@ -230,9 +245,10 @@ __global__ void __launch_bounds__(256) capped_attn_mfma_kernel(
 #pragma unroll
       for (int rr = 0; rr < 4; ++rr) {
         const int kk = k0 + g * 8 + h2 * 4 + rr;     // key of C row g*4+rr
-        float sv = sacc[rr] * scale;
+        float sv = sacc[rr] * scale * hs;
         if (cap > 0.f) sv = cap * cm_tanh(sv * inv_cap);
-        sc[h2 * 4 + rr] = (kk < limit && kk >= lo) ? sv : -INFINITY;
+        sc[h2 * 4 + rr] =
+            (kk < limit && (kk >= lo || kk < keep_first)) ? sv : -INFINITY;
       }
     }
     float mloc = sc[0];
@@ -372,7 +388,8 @@ void launch_capped_attn_mfma(float* out, float* ws_acc, float* ws_ml,
                              int heads, int n_kv, int D, int Dv,
                              int block_size, int table_width, float scale,
                              float cap, long q_stride, int n_part, int window,
-                             const float* sink, hipStream_t st) {
+                             const float* sink, int keep_first,
+                             const float* head_scale, hipStream_t st) {
   if (tokens == 0) return;
   const int cls = capped_attn_mfma_class(D, Dv);
   const int per = heads / n_kv;
@@ -390,7 +407,8 @@ void launch_capped_attn_mfma(float* out, float* ws_acc, float* ws_ml,
                      (size_t)(KQ * 2 + NO) * 1024, st, out, ws_acc, ws_ml,   \
                      q, k_cache, v_cache, block_tables, cu_q, seq_lens,      \
                      n_seqs, heads, n_kv, D, Dv, block_size, table_width,    \
-                     scale, cap, q_stride, n_part, window, sink)
+                     scale, cap, q_stride, n_part, window, sink, keep_first, \
+                     head_scale)
 #define CM_BY_CS(KQ, NO)                                                     \
   do {                                                                       \
     if (cs == 4) CM_LAUNCH(KQ, NO, 4);                                       \

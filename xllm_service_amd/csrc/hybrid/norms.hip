@@ -136,30 +136,42 @@ __global__ void gated_group_norm_kernel(
 }
 
 // res[row] += y[row] / rms(y[row]) * w1, and the new residual row once more
-// in the activation type (the operand of the next sublayer's GEMM)
-template <typename T>
+// in the activation type (the operand of the next sublayer's GEMM): as it
+// is, or with w_next normed for that sublayer, res / rms(res) * w_next. y may
+// be fp32 (a sum formed in fp32) or the activation type.
+template <typename TY, typename T>
 __global__ void norm_residual_add_kernel(float* __restrict__ res,
                                          T* __restrict__ h,
-                                         const T* __restrict__ y,
+                                         const TY* __restrict__ y,
                                          const float* __restrict__ w1,
-                                         float eps, int width, long y_stride) {
+                                         float eps, int width, long y_stride,
+                                         const float* __restrict__ w_next) {
   __shared__ float tmp[16];
   const int row = blockIdx.x;
-  const T* yr = y + (long)row * y_stride;
+  const TY* yr = y + (long)row * y_stride;
   float* rr = res + (long)row * width;
   T* hr = h + (long)row * width;
   float ss = 0.f;
   for (int i = threadIdx.x; i < width; i += blockDim.x) {
-    const float v = IO<T>::ld(yr + i);
+    const float v = IO<TY>::ld(yr + i);
     ss += v * v;
   }
   ss = block_reduce_sum(ss, tmp);
   const float rs = 1.0f / sqrtf(ss / (float)width + eps);
+  float s2 = 0.f;
   for (int i = threadIdx.x; i < width; i += blockDim.x) {
-    const float v = rr[i] + IO<T>::ld(yr + i) * rs * w1[i];
+    const float v = rr[i] + IO<TY>::ld(yr + i) * rs * w1[i];
     rr[i] = v;
-    IO<T>::st(hr + i, v);
+    s2 += v * v;
+    if (w_next == nullptr) IO<T>::st(hr + i, v);
   }
+  if (w_next == nullptr) return;
+  __syncthreads();
+  s2 = block_reduce_sum(s2, tmp);
+  const float r2 = 1.0f / sqrtf(s2 / (float)width + eps);
+  // a thread reads back the entries it wrote itself
+  for (int i = threadIdx.x; i < width; i += blockDim.x)
+    IO<T>::st(hr + i, rr[i] * r2 * w_next[i]);
 }
 
 XLLM_DEV float gelu_tanhf_(float z) {
@@ -237,13 +249,13 @@ void launch_norm_sigmoid_gate(T* out, const float* o, const float* w,
   hipLaunchKernelGGL((norm_sigmoid_gate_kernel<T>), dim3(rows), dim3(256), 0,
                      st, out, o, w, gate, eps, n, gate_stride, gate_cols);
 }
-template <typename T>
-void launch_norm_residual_add(float* res, T* h, const T* y, const float* w1,
+template <typename TY, typename T>
+void launch_norm_residual_add(float* res, T* h, const TY* y, const float* w1,
                               float eps, int rows, int width, long y_stride,
-                              hipStream_t st) {
+                              const float* w_next, hipStream_t st) {
   if (rows == 0) return;
-  hipLaunchKernelGGL((norm_residual_add_kernel<T>), dim3(rows), dim3(256), 0,
-                     st, res, h, y, w1, eps, width, y_stride);
+  hipLaunchKernelGGL((norm_residual_add_kernel<TY, T>), dim3(rows), dim3(256),
+                     0, st, res, h, y, w1, eps, width, y_stride, w_next);
 }
 template <typename T>
 void launch_gated_group_norm(T* out, const float* o, const float* w,
@@ -289,9 +301,6 @@ void launch_rope_interleaved(T* x, const long* pos, const double* inv_freq,
   template void launch_norm_sigmoid_gate<T>(T*, const float*, const float*,   \
                                             const T*, float, int, int, long,  \
                                             int, hipStream_t);                \
-  template void launch_norm_residual_add<T>(float*, T*, const T*,             \
-                                            const float*, float, int, int,    \
-                                            long, hipStream_t);               \
   template void launch_silu_mul<T>(T*, const T*, long, int, hipStream_t);     \
   template void launch_gelu_tanh_mul<T>(T*, const T*, long, int,              \
                                         hipStream_t);                         \
@@ -303,6 +312,14 @@ void launch_rope_interleaved(T* x, const long* pos, const double* inv_freq,
                                            int, hipStream_t);
 INST_NORMS(float)
 INST_NORMS(unsigned short)
+
+#define INST_NRA(TY, T)                                                      \
+  template void launch_norm_residual_add<TY, T>(                             \
+      float*, T*, const TY*, const float*, float, int, int, long,            \
+      const float*, hipStream_t);
+INST_NRA(float, float)
+INST_NRA(float, unsigned short)
+INST_NRA(unsigned short, unsigned short)
 
 #define INST_GRN(TI, TO)                                                     \
   template void launch_group_rmsnorm<TI, TO>(TO*, const TI*, const float*,   \
