@@ -288,3 +288,154 @@ def forward(cfg, weights, tokens, dtype=torch.float64):
         after.append(x)
     hid = rms_norm(x, w["final.norm"], cfg["norm"]["eps"])
     return hid @ w["embed"].T, torch.stack(after)
+
+
+# ---- test models: configurations, random checkpoints, model folders ---------
+def attn(kind="attention", heads=4, kv_heads=2, dim=8, vdim=8, dims=4,
+         base=100.0, scaling=None, size=5, keep_first=2, scale=None, mlp=12):
+    """One layer entry. mlp: int = dense feed-forward of that size, dict =
+    as given, None = none. size None = no mask."""
+    m = dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim,
+             scale=scale if scale is not None else dim ** -0.5)
+    if kind != "attention_2" and dims:
+        m["rot"] = dict(base=base, dims=dims)
+        if scaling:
+            m["rot"]["scaling"] = scaling
+    if kind != "attention_3" and size is not None:
+        m["mask"] = dict(size=size, keep_first=keep_first)
+    if kind == "attention_2":
+        m["vdim"] = dim
+    if isinstance(mlp, int):
+        mlp = dict(kind="dense", ff=mlp)
+    return dict(type=kind, mixer=m, mlp=mlp)
+
+
+def moe(ff=6, experts=4, top=2, identity=2, groups=(3, 2), shared=5):
+    r = dict(experts=experts, top=top, identity=identity)
+    if groups:
+        r["groups"] = dict(count=groups[0], keep=groups[1])
+    d = dict(kind="moe", expert=dict(ff=ff), router=r)
+    if shared:
+        d["shared"] = dict(ff=shared)
+    return d
+
+
+def make_config(width=24, vocab=50, eps=1e-5, mult=0.4, side=3, loop=None,
+                layers=None):
+    d = dict(architecture="Gararax", vocab=vocab, width=width,
+             norm=dict(eps=eps), residual_mult=mult,
+             layers=layers or [attn("attention_2"), attn("attention_3"),
+                               attn("attention")])
+    if side:
+        d["token_side"] = dict(dim=side)
+    if loop:
+        d["loop"] = dict(start=loop[0], stop=loop[1], times=loop[2])
+    return d
+
+
+def make_weights(cfg, seed=0, gain=1.0):
+    """Random bf16-representable weights (fp32 tensors) for a config."""
+    g = torch.Generator().manual_seed(seed)
+    W, n = cfg["width"], len(cfg["layers"])
+
+    def rnd(*shape, std=None):
+        std = std if std is not None else gain / math.sqrt(shape[-1])
+        return (torch.randn(*shape, generator=g) * std).bfloat16().float()
+
+    def near_one(k, spread=0.2):
+        return (1.0 + spread * torch.randn(k, generator=g)).bfloat16().float()
+
+    out = {"embed": rnd(cfg["vocab"], W, std=1.0), "final.norm": near_one(W)}
+    side = (cfg.get("token_side") or {}).get("dim", 0)
+    if side:
+        out["side.embed"] = rnd(cfg["vocab"], n * side, std=1.0)
+    lp = cfg.get("loop")
+    if lp and lp["stop"] > lp["start"]:
+        out["loop.step"] = rnd(lp["times"], W, std=0.5)
+    for i, lc in enumerate(cfg["layers"]):
+        p = f"l{i}."
+        mc, m = lc["mixer"], p + "mix."
+        H, G, D, Dv = mc["heads"], mc["kv_heads"], mc["dim"], mc["vdim"]
+        for nm in ("norm1", "norm1b"):
+            out[p + nm] = near_one(W)
+        # queries and keys large enough for a peaked softmax
+        out[m + "q"], out[m + "k"] = rnd(H * D, W, std=1.5 / math.sqrt(W)), \
+            rnd(G * D, W, std=1.5 / math.sqrt(W))
+        if lc["type"] != "attention_2":
+            out[m + "v"] = rnd(G * Dv, W)
+        else:
+            out[m + "g"] = rnd(H * Dv, W)
+        if lc["type"] == "attention_3":
+            out[m + "q.b"], out[m + "k.b"] = rnd(H * D, std=0.3), \
+                rnd(G * D, std=0.3)
+            out[m + "v.b"] = rnd(G * Dv, std=0.3)
+            out[m + "temp"] = near_one(H, 0.4)
+        out[m + "o"] = rnd(W, H * Dv)
+        mlp, f = lc.get("mlp"), p + "mlp."
+        if mlp:
+            for nm in ("norm2", "norm2b"):
+                out[p + nm] = near_one(W)
+            if mlp["kind"] == "dense":
+                out[f + "up"], out[f + "down"] = rnd(mlp["ff"], W), \
+                    rnd(W, mlp["ff"])
+                out[f + "act"] = rnd(4, std=0.7)
+            else:
+                r = mlp["router"]
+                n_all = r["experts"] + r.get("identity", 0)
+                out[f + "router"] = rnd(n_all, W, std=2.0 / math.sqrt(W))
+                # corrections comparable to the scores, of both signs
+                out[f + "correction"] = rnd(n_all, std=0.5 / n_all)
+                ff = mlp["expert"]["ff"]
+                for j in range(r["experts"]):
+                    e = f"{f}e{j}."
+                    out[e + "gate"], out[e + "up"] = rnd(ff, W), rnd(ff, W)
+                    out[e + "down"] = rnd(W, ff)
+                if mlp.get("shared"):
+                    sf = mlp["shared"]["ff"]
+                    out[f + "shared.gate"] = rnd(sf, W)
+                    out[f + "shared.up"] = rnd(sf, W)
+                    out[f + "shared.down"] = rnd(W, sf)
+        if side:
+            out[p + "side.gate"], out[p + "side.proj"] = rnd(side, W), \
+                rnd(W, side)
+            out[p + "side.norm"] = near_one(W)
+    return out
+
+
+def write_safetensors(path, tensors):
+    """bf16 file: 8-byte header length, JSON header, raw data."""
+    import json
+    import struct
+    header, blobs, at = {}, [], 0
+    for name, t in tensors.items():
+        raw = t.to(torch.bfloat16).contiguous().view(torch.int16).numpy() \
+            .tobytes()
+        header[name] = dict(dtype="BF16", shape=list(t.shape),
+                            data_offsets=[at, at + len(raw)])
+        blobs.append(raw)
+        at += len(raw)
+    js = json.dumps(header).encode()
+    with open(path, "wb") as f:
+        f.write(struct.pack("<Q", len(js)))
+        f.write(js)
+        for b in blobs:
+            f.write(b)
+
+
+def write_model_dir(folder, cfg, weights):
+    import json
+    import os
+    os.makedirs(folder, exist_ok=True)
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    write_safetensors(os.path.join(folder, "model.safetensors"), weights)
+    return folder
+
+
+def rel_err(got, want):
+    """Per row: rms of the mean-free difference over the rms of `want`."""
+    got, want = got.to(torch.float64), want.to(torch.float64)
+    d = got - want
+    d = d - d.mean(-1, keepdim=True)
+    ref = want - want.mean(-1, keepdim=True)
+    return torch.sqrt((d ** 2).mean(-1)) / torch.sqrt((ref ** 2).mean())
