@@ -67,7 +67,7 @@ def parse_args():
                          "measurement, not the headline record)")
     ap.add_argument("--hybrid-sizes", default="2k,4k")
     ap.add_argument("--hybrid-family", default="pugovik",
-                    choices=("pugovik", "dunusun", "tosipel"),
+                    choices=("pugovik", "dunusun", "tosipel", "gararax"),
                     help="which hybrid stack --mode hybrid measures beside "
                          "the equal-size llama stack")
     ap.add_argument("--model", default="llama-3-8b")
@@ -565,6 +565,169 @@ def _tosipel_kernels(size, device, T, batch, ctx):
     return out
 
 
+def _gararax_kernels(size, device, T, batch, ctx):
+    """Achieved rates of the Gararax kernels at one layer's shapes, beside
+    the like kernels of the tosipel / pugovik / llama stacks of that size."""
+    from xllm_service_amd import ops
+    from xllm_service_amd.models.config import get_config
+    from xllm_service_amd.ops import hybrid as hops
+    gc, tc, pc, lc = (get_config(f"{f}-{size}") for f in (
+        "gararax", "tosipel", "pugovik", "llama"))
+    a1 = next(l.mixer for l in gc.layers if l.type == "attention")
+    a2 = next(l.mixer for l in gc.layers if l.type == "attention_2")
+    a3 = next(l.mixer for l in gc.layers if l.type == "attention_3")
+    moe = next(l.mlp for l in gc.layers if l.mlp["kind"] == "moe")
+    dense = next(l.mlp for l in gc.layers if l.mlp["kind"] == "dense")
+    tatt = next(l.mixer for l in tc.layers if l.type == "attention")
+    pmoe = next(l.mlp for l in pc.layers if l.mlp)
+    bf = dict(dtype=torch.bfloat16, device=device)
+    f32 = dict(dtype=torch.float32, device=device)
+    i32 = dict(dtype=torch.int32, device=device)
+    out = []
+    nblk = (max(T, ctx) + 15) // 16
+    tab = torch.arange(batch * nblk, **i32).view(batch, nblk)
+    cu = torch.tensor([0, T], **i32)
+    sl = torch.tensor([T], **i32)
+    sld = torch.full((batch,), ctx, **i32)
+
+    def attn_pair(label, m, window, keep, sink, hs, same, tail=""):
+        H, G, D, Dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+        kc = torch.randn(batch * nblk, G, 16, D, **bf)
+        vc = kc if same else torch.randn(batch * nblk, G, 16, Dv, **bf)
+        q = torch.randn(T, H * D, **bf)
+        o = torch.empty(T, H, Dv, **f32)
+        sk = torch.zeros(H, **f32) if sink else None
+        hsc = torch.ones(H, **f32) if hs else None
+        kw = dict(window=window, sink=sk, keep_first=keep, head_scale=hsc)
+        seen = sum(min(i + 1, window) + min(keep, max(i + 1 - window, 0))
+                   if window else i + 1 for i in range(T))
+        t = _time_gpu(lambda: hops.capped_attn(q, kc, vc, tab[:1], cu, sl, H,
+                                               m["scale"], 0.0, o, **kw), 3, 1)
+        out.append((f"{label} prefill{tail}", t,
+                    2.0 * H * (D + Dv) * seen / t / 1e12, "TFLOP/s"))
+        qd = torch.randn(batch, H * D, **bf)
+        od = torch.empty(batch, H, Dv, **f32)
+        t = _time_gpu(lambda: hops.capped_attn(qd, kc, vc, tab, None, sld, H,
+                                               m["scale"], 0.0, od, **kw))
+        keys = min(ctx, window + keep) if window else ctx
+        width = D if same else D + Dv
+        out.append((f"{label} decode{tail}", t,
+                    batch * keys * G * width * 2 / t / 1e9, "GB/s"))
+
+    w1 = a1["mask"]
+    attn_pair("window+kept attn", a1, w1["size"], w1["keep_first"], False,
+              False, False, f" (window {w1['size']}, kept {w1['keep_first']})")
+    w2 = a2["mask"]
+    attn_pair("keys-as-values sink attn", a2, w2["size"], w2["keep_first"],
+              True, False, True, f" (window {w2['size']})")
+    attn_pair("full attn, head multiplier", a3, 0, 0, False, True, False)
+    attn_pair("window+sink attn (tosipel)", tatt, tatt["mask"]["size"], 0,
+              True, False, False, f" (window {tatt['mask']['size']})")
+    Hq, Hk, Dl = lc.num_heads, lc.num_kv_heads, lc.head_dim
+    kl = torch.randn(batch * nblk, Hk, 16, Dl, **bf)
+    vl = torch.randn(batch * nblk, Hk, 16, Dl, **bf)
+    if Dl == 128:
+        ql = torch.randn(T, Hq, Dl, **bf)
+        t = _time_gpu(lambda: ops.paged_attn_prefill(ql, kl, vl, tab[:1], cu,
+                                                     sl, 0.1), 3, 1)
+        out.append(("paged_attn prefill (llama)", t,
+                    4.0 * Hq * Dl * T * (T + 1) / 2 / t / 1e12, "TFLOP/s"))
+    qld = torch.randn(batch, Hq, Dl, **bf)
+    t = _time_gpu(lambda: ops.paged_attn_decode(qld, kl, vl, tab, sld, 0.1))
+    out.append(("paged_attn decode (llama)", t,
+                batch * ctx * Hk * Dl * 2 * 2 / t / 1e9, "GB/s"))
+    # ---- query/key preparation with paged store ----------------------------
+    H, G, D, Dv = a1["heads"], a1["kv_heads"], a1["dim"], a1["vdim"]
+    rot = a1["rot"]["dims"]
+    proj = torch.randn(T, H * D + G * D + G * Dv, **bf)
+    kc = torch.zeros(nblk, G, 16, D, **bf)
+    vc = torch.zeros(nblk, G, 16, Dv, **bf)
+    pos = torch.arange(T, dtype=torch.long, device=device)
+    inv = torch.rand(rot // 2, dtype=torch.float64, device=device)
+    nbytes = T * (2 * H * D + 2 * G * D + 2 * G * Dv) * 2
+    t = _time_gpu(lambda: hops.rope_headnorm_store(
+        proj[:, :H * D], proj[:, H * D:H * D + G * D], proj[:, H * D + G * D:],
+        pos, inv, rot, True, True, 1e-6, H, G, kc, vc, pos))
+    out.append(("rope_headnorm_store", t, nbytes / t / 1e9, "GB/s"))
+    Ht, Gt, Dt, Dvt = tatt["heads"], tatt["kv_heads"], tatt["dim"], \
+        tatt["vdim"]
+    rt = tatt["rot"]["dims"]
+    projt = torch.randn(T, Ht * Dt + Gt * Dt + Gt * Dvt, **bf)
+    kct = torch.zeros(nblk, Gt, 16, Dt, **bf)
+    vct = torch.zeros(nblk, Gt, 16, Dvt, **bf)
+    invt = torch.rand(rt // 2, dtype=torch.float64, device=device)
+    wq, wk = torch.ones(Ht * Dt, **f32), torch.ones(Gt * Dt, **f32)
+    t = _time_gpu(lambda: hops.rownorm_rope_store(
+        projt[:, :Ht * Dt], projt[:, Ht * Dt:Ht * Dt + Gt * Dt],
+        projt[:, Ht * Dt + Gt * Dt:], wq, wk, 1e-6, pos, invt, rt, Ht, Gt,
+        kct, vct, pos))
+    out.append(("rownorm_rope_store (tosipel)", t,
+                T * (2 * Ht * Dt + 2 * Gt * Dt + 2 * Gt * Dvt) * 2 / t / 1e9,
+                "GB/s"))
+    # ---- norms and activations ---------------------------------------------
+    Wd = gc.hidden_size
+    x = torch.randn(T, Wd, **f32)
+    w = torch.ones(Wd, **f32)
+    y = torch.randn(T, Wd, **bf)
+    y32 = torch.randn(T, Wd, **f32)
+    t = _time_gpu(lambda: hops.norm_residual_add_(x, y, w, 1e-6,
+                                                  torch.bfloat16, w))
+    out.append(("norm_residual_add + next norm", t, T * Wd * 12 / t / 1e9,
+                "GB/s"))
+    t = _time_gpu(lambda: hops.norm_residual_add_(x, y32, w, 1e-6,
+                                                  torch.bfloat16, w))
+    out.append(("norm_residual_add + next norm (fp32 input)", t,
+                T * Wd * 14 / t / 1e9, "GB/s"))
+    t = _time_gpu(lambda: hops.norm_residual_add_(x, y, w, 1e-6,
+                                                  torch.bfloat16))
+    out.append(("norm_residual_add (tosipel)", t, T * Wd * 12 / t / 1e9,
+                "GB/s"))
+    ff = dense["ff"]
+    z = torch.randn(T, ff, **bf)
+    coef = torch.tensor([0.5, 0.3, 0.2, 0.0], **f32)
+    t = _time_gpu(lambda: hops.polynorm(z, coef, 1e-6))
+    out.append(("polynorm", t, T * ff * 4 / t / 1e9, "GB/s"))
+    z2 = torch.randn(T, 2 * ff, **bf)
+    t = _time_gpu(lambda: hops.gelu_tanh_mul(z2))
+    out.append(("gelu_tanh_mul (tosipel)", t, T * ff * 6 / t / 1e9, "GB/s"))
+    sd = gc.side_dim
+    ga = torch.randn(T, sd, **bf)
+    tbl = torch.randn(T, sd * gc.num_layers, **bf)
+    t = _time_gpu(lambda: hops.gelu_tanh_gate(ga, tbl[:, sd:2 * sd]))
+    out.append(("gelu_tanh_gate (side input)", t, T * sd * 6 / t / 1e9,
+                "GB/s"))
+    # ---- router and combine --------------------------------------------------
+    r = moe["router"]
+    n_all = r["experts"] + r["identity"]
+    h = torch.randn(T, Wd, **bf)
+    wr = torch.randn(n_all, Wd, **f32)
+    corr = torch.zeros(n_all, **f32)
+    t = _time_gpu(lambda: hops.moe_route(
+        h, wr, r["top"], r["groups"]["count"], r["groups"]["keep"],
+        softmax=True, correction=corr, group_max=True, normalize=True))
+    out.append(("moe_route softmax+correction", t, T / t / 1e6, "Mtok/s"))
+    pr = pmoe["router"]
+    wrp = torch.randn(pr["experts"], pc.hidden_size, **f32)
+    hp = torch.randn(T, pc.hidden_size, **bf)
+    t = _time_gpu(lambda: hops.moe_route(hp, wrp, pr["top"],
+                                         pr["groups"]["count"],
+                                         pr["groups"]["keep"]))
+    out.append(("moe_route sigmoid (pugovik)", t, T / t / 1e6, "Mtok/s"))
+    top = r["top"]
+    ye = torch.randn(T * top, Wd, **bf)
+    rows = torch.arange(T * top, **i32).view(T, top).clone()
+    rows[::3, 0] = -1
+    wts = torch.rand(T, top, **f32)
+    t = _time_gpu(lambda: hops.moe_combine(ye, rows, wts, T, h, y))
+    out.append(("moe_combine + identity + shared", t,
+                T * Wd * (2 * top + 2 + 4) / t / 1e9, "GB/s"))
+    rows0 = torch.arange(T * top, **i32).view(T, top)
+    t = _time_gpu(lambda: hops.moe_combine(ye, rows0, wts, T))
+    out.append(("moe_combine (pugovik)", t, T * Wd * (2 * top + 4) / t / 1e9,
+                "GB/s"))
+    return out
+
+
 def run_hybrid_mode(args, device):
     assert torch.cuda.is_available(), "hybrid mode measures the HIP path"
     kernels = _hybrid_kernels
@@ -575,6 +738,9 @@ def run_hybrid_mode(args, device):
     if args.hybrid_family == "tosipel":
         kernels = _tosipel_kernels
         fams = ("tosipel", "dunusun", "llama")
+    if args.hybrid_family == "gararax":
+        kernels = _gararax_kernels
+        fams = ("gararax", "tosipel", "pugovik", "llama")
     for size in args.hybrid_sizes.split(","):
         T, batch, ctx = 4096, 32, 2048
         for name, t, rate, unit in kernels(size, device, T, batch, ctx):

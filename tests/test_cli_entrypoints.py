@@ -22,7 +22,7 @@ def _free_port():
 
 @pytest.mark.timeout(180)
 @pytest.mark.parametrize("model", ["llama-tiny", "dunusun-tiny",
-                                   "tosipel-tiny"])
+                                   "tosipel-tiny", "gararax-tiny"])
 def test_master_and_worker_cli(model):
     http_port, rpc_port, reg_port = _free_port(), _free_port(), _free_port()
     env = dict(os.environ)

@@ -30,6 +30,10 @@
 // (k>>3)*64 + (k&3)*16 + (d&15); a lane reads 8 B at g*128 + n*8 (bytes) of
 // each 512-byte half.
 //
+// Keys read as values (v_cache is the very tensor k_cache): the key image of
+// a tile is also its value image (both have one layout), so the tile is
+// fetched and staged once.
+//
 // Decode splits the context over `n_part` workgroups per (token, key/value
 // head); partial (acc, max, sum) triples are merged by a second small kernel.
 //
@@ -88,8 +92,11 @@ __global__ void __launch_bounds__(256) capped_attn_mfma_kernel(
   constexpr int NPV = NB;                         // 16 B value chunks per thread
   constexpr bool PF = CS > 1;
   constexpr int Dp = KQ * 32, Dvp = NO * 16;
+  // keys read as values: one image (the instantiations with D == Dv have
+  // Dp == Dvp)
+  const bool same = (k_cache == v_cache) && Dp == Dvp;
   unsigned short* kt = cm_lds;                    // key image: Dp/16 tiles
-  unsigned short* vt = cm_lds + (Dp / 16) * 512;  // value image: NO tiles
+  unsigned short* vt = same ? kt : cm_lds + (Dp / 16) * 512;  // NO tiles
   const int per = heads / n_kv;
   const int kvh = blockIdx.z;
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
@@ -200,8 +207,10 @@ __global__ void __launch_bounds__(256) capped_attn_mfma_kernel(
   if (PF && i_begin < i_end) {
 #pragma unroll
     for (int i = 0; i < NPK; ++i) prek[i] = fetch(k_cache, D, CHK, t_begin, i);
+    if (!same) {
 #pragma unroll
-    for (int i = 0; i < NPV; ++i) prev[i] = fetch(v_cache, Dv, CHV, t_begin, i);
+      for (int i = 0; i < NPV; ++i) prev[i] = fetch(v_cache, Dv, CHV, t_begin, i);
+    }
   }
 
   for (int it = i_begin; it < i_end; ++it) {
@@ -211,21 +220,27 @@ __global__ void __launch_bounds__(256) capped_attn_mfma_kernel(
     if (PF) {
 #pragma unroll
       for (int i = 0; i < NPK; ++i) put(kt, CHK, i, prek[i]);
+      if (!same) {
 #pragma unroll
-      for (int i = 0; i < NPV; ++i) put(vt, CHV, i, prev[i]);
+        for (int i = 0; i < NPV; ++i) put(vt, CHV, i, prev[i]);
+      }
     } else {
 #pragma unroll
       for (int i = 0; i < NPK; ++i) put(kt, CHK, i, fetch(k_cache, D, CHK, t, i));
+      if (!same) {
 #pragma unroll
-      for (int i = 0; i < NPV; ++i) put(vt, CHV, i, fetch(v_cache, Dv, CHV, t, i));
+        for (int i = 0; i < NPV; ++i) put(vt, CHV, i, fetch(v_cache, Dv, CHV, t, i));
+      }
     }
     __syncthreads();
     if (PF && it + 1 < i_end) {         // next tile flies during the compute
       const int tn = tile_at(it + 1);
 #pragma unroll
       for (int i = 0; i < NPK; ++i) prek[i] = fetch(k_cache, D, CHK, tn, i);
+      if (!same) {
 #pragma unroll
-      for (int i = 0; i < NPV; ++i) prev[i] = fetch(v_cache, Dv, CHV, tn, i);
+        for (int i = 0; i < NPV; ++i) prev[i] = fetch(v_cache, Dv, CHV, tn, i);
+      }
     }
     if (!wave_on) continue;
     // ---- scores ------------------------------------------------------------

@@ -205,6 +205,8 @@ class GararaxForCausalLM(nn.Module):
             put(self.side_embed.weight, take("side.embed"))
         if self.looped:
             put(self.loop_step, take("loop.step"))
+        else:
+            used.add("loop.step")          # a loop over no layers adds nothing
         for i, blk in enumerate(self.blocks):
             p = f"l{i}."
             m, mx = p + "mix.", blk.mixer
