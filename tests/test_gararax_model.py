@@ -72,10 +72,10 @@ def _variants():
                  keep_first=4, mlp=192),
             attn("attention", heads=2, kv_heads=1, dim=128, vdim=80, dims=64,
                  base=500.0, scaling=BAND, size=40, keep_first=35,
-                 mlp=moe(ff=48, experts=8, top=4, identity=4, groups=(4, 3),
+                 mlp=moe(ff=48, experts=9, top=3, identity=3, groups=(4, 2),
                          shared=64)),
-            attn("attention_3", heads=4, kv_heads=1, dim=128, vdim=32,
-                 dims=64, base=10000.0, mlp=moe(ff=32, experts=5, top=2,
+            attn("attention_3", heads=4, kv_heads=2, dim=128, vdim=48,
+                 dims=32, base=10000.0, mlp=moe(ff=32, experts=5, top=2,
                                                 identity=0, groups=None,
                                                 shared=16))]),
     }

@@ -209,7 +209,7 @@ def _attn_case(target, H, G, D, Dv, L, n_q, window, keep, standout, seed,
     return out, want
 
 
-SHAPES = [(4, 2, 8, 6), (6, 2, 64, 64), (4, 1, 128, 32), (2, 2, 64, 80),
+SHAPES = [(4, 2, 8, 6), (6, 2, 64, 64), (4, 1, 128, 48), (2, 2, 64, 80),
           (3, 3, 10, 10)]
 
 
@@ -272,7 +272,7 @@ def test_zero_sink_keys_as_values_and_head_multiplier(target, decode):
     g2, w2 = _attn_case(target, 4, 2, 64, 64, 5, 5, 3, 1, None, 7, same=True,
                         decode=decode)
     assert float((w2 - want).abs().max()) > 0.05      # the sink matters
-    got, want = _attn_case(target, 4, 1, 128, 32, 70, 4, 0, 0, None, 8,
+    got, want = _attn_case(target, 4, 1, 128, 48, 70, 4, 0, 0, None, 8,
                            temp=True, decode=decode)
     _close(got, want, target, "multiplier")
     got, want = _attn_case(target, 3, 3, 10, 10, 40, 4, 9, 2, 31, 9,
@@ -334,7 +334,7 @@ def _route_case(g, T, W, experts, identity, top, groups, corr_scale):
 
 @pytest.mark.parametrize("target", TARGETS)
 @pytest.mark.parametrize("experts,identity,top,groups,corr", [
-    (8, 4, 4, (4, 3), 0.05), (6, 0, 2, None, 0.0), (5, 1, 1, (3, 1), 0.3),
+    (10, 2, 3, (4, 2), 0.05), (6, 0, 2, None, 0.0), (5, 1, 1, (3, 1), 0.3),
     (16, 0, 3, (4, 1), 2.0), (64, 8, 6, (8, 4), 0.01), (3, 0, 3, None, 0.1)])
 def test_router(target, experts, identity, top, groups, corr):
     """Softmax scores, choice on score + correction (strongly negative
