@@ -71,8 +71,13 @@ XLLM_DEV float cm_tanh(float x) {          // 1 - 2 / (e^(2x) + 1)
 // value row (Dv padded to 64). CS = column split: the 4 waves of a workgroup
 // form 4/CS row tiles, and CS waves share one row tile, each owning every
 // CS-th 64-column batch of the output (decode: few rows per token).
+// The decode instantiation for 128-wide heads sits at the edge of four waves
+// per SIMD (128 registers); the second launch bound asks the compiler to stay
+// inside it (0 = no request).
 template <int KQ, int NO, int CS>
-__global__ void __launch_bounds__(256) capped_attn_mfma_kernel(
+__global__ void
+__launch_bounds__(256, (KQ == 4 && NO == 8 && CS == 4) ? 4 : 0)
+capped_attn_mfma_kernel(
     float* __restrict__ out, float* __restrict__ ws_acc,
     float* __restrict__ ws_ml, const unsigned short* __restrict__ q,
     const unsigned short* __restrict__ k_cache,
