@@ -18,7 +18,7 @@ from xllm_service_amd.engine.sampling import SamplingParams
 TARGETS = [("cpu", torch.float32),
            pytest.param(("cuda", torch.float32), marks=pytest.mark.gpu),
            pytest.param(("cuda", torch.bfloat16), marks=pytest.mark.gpu)]
-BAND = dict(factor=4.0, low=1.0, high=4.0, original=64)
+BAND = dict(factor=8.0, low=1.0, high=2.0, original=48)
 
 
 def _variants():

@@ -209,7 +209,7 @@ def _attn_case(target, H, G, D, Dv, L, n_q, window, keep, standout, seed,
     return out, want
 
 
-SHAPES = [(4, 2, 8, 6), (6, 2, 64, 64), (4, 1, 128, 48), (2, 2, 64, 80),
+SHAPES = [(4, 2, 8, 6), (6, 2, 64, 64), (4, 1, 128, 48), (2, 2, 64, 72),
           (3, 3, 10, 10)]
 
 
