@@ -244,7 +244,7 @@ def test_a_far_kept_key_decides():
 
 
 @pytest.mark.parametrize("target", TARGETS)
-@pytest.mark.parametrize("name", ["mixed", "looped"])
+@pytest.mark.parametrize("name", ["mixed", "looped", "large"])
 def test_unequal_batch_with_reused_pages(root, target, name):
     """A pool far smaller than the sum of all requests: requests come and go
     in mixed batches (prompt portions beside single tokens), later ones land
